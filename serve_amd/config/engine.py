@@ -1,0 +1,48 @@
+"""Engine settings.  The reference keeps these as literals in code: page size 64
+(serve/run.py:247), 2048 prompt tokens per prefill step (serve/run.py:265), the 0.9
+admission factor (serve/run.py:277), 0.6 of free memory for the cache (serve/model.py:172),
+4000 requests (serve/run.py:13), a context of 2048 (serve/model.py:32).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+DTYPES = ("bfloat16", "float32")
+
+
+@dataclass
+class EngineConfig:
+    dtype: str = "bfloat16"
+    page_size: int = 16
+    # size of the page pool: explicit, or a fraction of the free device memory
+    num_pages: Optional[int] = None
+    memory_fraction: float = 0.6
+    max_context: int = 4096
+    max_requests: int = 256
+    max_tokens_per_step: int = 2048
+    prefill_chunk: int = 2048
+    # "reserve": admit a request only if pages for prompt + max_new_tokens are free
+    # (what the reference's admission does, serve/run.py:273-280); "optimistic": pages as
+    # the request grows, and the youngest running request is preempted when they run out.
+    admission: str = "reserve"
+    seed: int = 0
+    device: str = "cuda:0"
+    # replay a decode-only step from a captured HIP graph
+    use_graphs: bool = True
+
+    def validate(self) -> None:
+        if self.dtype not in DTYPES:
+            raise ValueError(f"dtype must be one of {DTYPES}, got {self.dtype!r}")
+        if self.page_size <= 0 or self.page_size % 4:
+            raise ValueError(f"page_size must be a positive multiple of 4, got {self.page_size}")
+        if self.admission not in ("reserve", "optimistic"):
+            raise ValueError(f"admission must be 'reserve' or 'optimistic', got {self.admission!r}")
+        if self.max_context <= 0 or self.max_requests <= 0 or self.max_tokens_per_step <= 0:
+            raise ValueError("max_context, max_requests and max_tokens_per_step must be positive")
+        if self.prefill_chunk <= 0:
+            raise ValueError("prefill_chunk must be positive")
+
+    @property
+    def max_pages_per_request(self) -> int:
+        return -(-self.max_context // self.page_size)

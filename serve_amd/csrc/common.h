@@ -1,0 +1,76 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, wave reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define SA_WAVE 64
+
+// dtype codes of the C interface
+enum { SA_F32 = 0, SA_BF16 = 1 };
+
+// error codes of the C interface (0 = ok, >0 = hipError_t of the launch)
+enum { SA_ERR_ARG = -1, SA_ERR_UNSUPPORTED = -2 };
+
+struct bf16_t {
+  uint16_t v;
+};
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return bf16_bits_to_float(x.v); }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float x);
+template <>
+__device__ __forceinline__ float from_float<float>(float x) {
+  return x;
+}
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
+  bf16_t r;
+  r.v = float_to_bf16_bits(x);
+  return r;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = SA_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, SA_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = SA_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, SA_WAVE));
+  return v;
+}
+
+// sum over a block of up to 1024 threads; `scratch` holds at least 16 floats of LDS
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (SA_WAVE - 1);
+  const int wave = threadIdx.x / SA_WAVE;
+  const int nwaves = (blockDim.x + SA_WAVE - 1) / SA_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nwaves; ++i) t += scratch[i];
+  return t;
+}
+
+#define SA_LAUNCH_CHECK()                      \
+  do {                                         \
+    hipError_t e__ = hipGetLastError();        \
+    if (e__ != hipSuccess) return (int)e__;    \
+  } while (0)

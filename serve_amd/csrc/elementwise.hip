@@ -1,0 +1,193 @@
+// Row-wise kernels of the step: embedding gather, residual add + RMSNorm, rotation of q and k
+// with the write of k and v into cache pages, and the SwiGLU gate.  All arithmetic is fp32;
+// the template types are storage only.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// embedding: x[t, :] = table[tokens[t], :]   (serve/model.py:220), residual stream in fp32
+// ---------------------------------------------------------------------------------------------
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ x, int d) {
+  const int t = blockIdx.x;
+  const size_t row = (size_t)tokens[t] * (size_t)d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) x[(size_t)t * d + i] = to_float(table[row + i]);
+}
+
+extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, float* x, int T, int d,
+                        hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (d <= 0) return SA_ERR_ARG;
+  dim3 grid(T), block(256);
+  if (table_dtype == SA_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, x, d);
+  else if (table_dtype == SA_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, x, d);
+  else
+    return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// residual add + RMSNorm (serve/model.py:63-68,147-148):
+//   v = x[t] + delta[t];  x[t] = v (only when rows == nullptr);  y[r] = v * rsqrt(mean(v^2) + eps) * w
+// rows != nullptr: output row r takes source row rows[r] and x is left untouched.
+// ---------------------------------------------------------------------------------------------
+template <typename TA, typename TW>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TA* __restrict__ delta,
+                                   const TW* __restrict__ w, TA* __restrict__ y,
+                                   const int* __restrict__ rows, float eps, int d) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int t = rows ? rows[r] : r;
+  float* xr = x + (size_t)t * d;
+  const TA* dr = delta ? delta + (size_t)t * d : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) {
+      v += to_float(dr[i]);
+      if (!rows) xr[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float rs = rsqrtf(ss / (float)d + eps);
+  TA* yr = y + (size_t)r * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];
+    if (dr && rows) v += to_float(dr[i]);
+    yr[i] = from_float<TA>((v * rs) * to_float(w[i]));
+  }
+}
+
+extern "C" int sa_add_rmsnorm(float* x, const void* delta, const void* w, int w_dtype, void* y,
+                              int act_dtype, const int* rows, float eps, int R, int d,
+                              hipStream_t stream) {
+  if (R <= 0) return 0;
+  if (d <= 0) return SA_ERR_ARG;
+  dim3 grid(R), block(d >= 1024 ? 256 : 64);
+#define GO(TA, TW)                                                                                \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TW>), grid, block, 0, stream, x, (const TA*)delta,  \
+                     (const TW*)w, (TA*)y, rows, eps, d)
+  if (act_dtype == SA_F32 && w_dtype == SA_F32) GO(float, float);
+  else if (act_dtype == SA_F32 && w_dtype == SA_BF16) GO(float, bf16_t);
+  else if (act_dtype == SA_BF16 && w_dtype == SA_F32) GO(bf16_t, float);
+  else if (act_dtype == SA_BF16 && w_dtype == SA_BF16) GO(bf16_t, bf16_t);
+  else return SA_ERR_UNSUPPORTED;
+#undef GO
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// rotation of q and k (serve/model.py:234-244) fused with the cache write
+// (serve/kernels/cache_write.py:49-165).
+//   qkv: [T, (Hq + 2 Hk) D]; q is rotated in place, rotated k and plain v go to the pages.
+//   angle = float(position) * inv_freq[j] in fp32, pair j = (j, j + rot/2) ("half") or
+//   (2j, 2j + 1) ("adjacent"); dims >= rot_dim pass through.
+//   k page layout [page, Hk, page_size, D]; v page layout [page, Hk, D, page_size].
+//   slot[t] = page * page_size + offset of token t, or < 0 for "do not store".
+// ---------------------------------------------------------------------------------------------
+template <typename TA, typename TC>
+__global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict__ positions,
+                                     const float* __restrict__ inv_freq, const int* __restrict__ slot,
+                                     TC* __restrict__ k_pages, TC* __restrict__ v_pages, int Hq, int Hk,
+                                     int D, int rot_dim, int adjacent, int page_size, int write_kv) {
+  const int t = blockIdx.x;
+  TA* row = qkv + (size_t)t * (size_t)(Hq + 2 * Hk) * D;
+  const float pos = (float)positions[t];
+  const int s = write_kv ? slot[t] : -1;
+  const int page = s >= 0 ? s / page_size : 0;
+  const int off = s >= 0 ? s % page_size : 0;
+  const int half = rot_dim / 2;
+
+  // rotated pairs of q heads and k heads
+  const int npairs = (Hq + Hk) * half;
+  for (int idx = threadIdx.x; idx < npairs; idx += blockDim.x) {
+    const int h = idx / half;
+    const int j = idx - h * half;
+    const int i0 = adjacent ? 2 * j : j;
+    const int i1 = adjacent ? 2 * j + 1 : j + half;
+    float sn, cs;
+    sincosf(pos * inv_freq[j], &sn, &cs);
+    TA* hp = row + (size_t)h * D;
+    const float a = to_float(hp[i0]);
+    const float b = to_float(hp[i1]);
+    const float o0 = a * cs - b * sn;
+    const float o1 = b * cs + a * sn;
+    if (h < Hq) {
+      hp[i0] = from_float<TA>(o0);
+      hp[i1] = from_float<TA>(o1);
+    } else if (s >= 0) {
+      TC* kp = k_pages + (((size_t)page * Hk + (h - Hq)) * page_size + off) * D;
+      kp[i0] = from_float<TC>(o0);
+      kp[i1] = from_float<TC>(o1);
+    }
+  }
+  if (s < 0) return;
+  // k dims that are not rotated
+  const int rest = D - rot_dim;
+  for (int idx = threadIdx.x; idx < Hk * rest; idx += blockDim.x) {
+    const int h = idx / rest;
+    const int i = rot_dim + (idx - h * rest);
+    TC* kp = k_pages + (((size_t)page * Hk + h) * page_size + off) * D;
+    kp[i] = from_float<TC>(to_float(row[(size_t)(Hq + h) * D + i]));
+  }
+  // v, stored transposed inside the page
+  for (int idx = threadIdx.x; idx < Hk * D; idx += blockDim.x) {
+    const int h = idx / D;
+    const int i = idx - h * D;
+    TC* vp = v_pages + (((size_t)page * Hk + h) * D + i) * page_size + off;
+    *vp = from_float<TC>(to_float(row[(size_t)(Hq + Hk + h) * D + i]));
+  }
+}
+
+extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, const float* inv_freq,
+                                const int* slot, void* k_pages, void* v_pages, int cache_dtype, int T,
+                                int Hq, int Hk, int D, int rot_dim, int adjacent, int page_size,
+                                int write_kv, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (Hq <= 0 || Hk < 0 || D <= 0 || rot_dim < 0 || rot_dim > D || (rot_dim & 1) || page_size <= 0)
+    return SA_ERR_ARG;
+  dim3 grid(T), block(256);
+#define GO(TA, TC)                                                                               \
+  hipLaunchKernelGGL((rope_kv_write_kernel<TA, TC>), grid, block, 0, stream, (TA*)qkv, positions, \
+                     inv_freq, slot, (TC*)k_pages, (TC*)v_pages, Hq, Hk, D, rot_dim, adjacent,   \
+                     page_size, write_kv)
+  if (act_dtype == SA_F32 && cache_dtype == SA_F32) GO(float, float);
+  else if (act_dtype == SA_BF16 && cache_dtype == SA_BF16) GO(bf16_t, bf16_t);
+  else return SA_ERR_UNSUPPORTED;
+#undef GO
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// SwiGLU gate (serve/model.py:85): a[t, i] = silu(gu[t, i]) * gu[t, I + i]
+// ---------------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ a, int T, int I) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  for (int t = blockIdx.y; t < T; t += gridDim.y) {
+    const float g = to_float(gu[(size_t)t * 2 * I + i]);
+    const float u = to_float(gu[(size_t)t * 2 * I + I + i]);
+    a[(size_t)t * I + i] = from_float<TA>((g / (1.f + expf(-g))) * u);
+  }
+}
+
+extern "C" int sa_silu_mul(const void* gu, void* a, int act_dtype, int T, int I, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (I <= 0) return SA_ERR_ARG;
+  dim3 grid((I + 255) / 256, T < 32768 ? T : 32768), block(256);
+  if (act_dtype == SA_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)a, T, I);
+  else if (act_dtype == SA_BF16)
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)a, T, I);
+  else
+    return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,272 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget, decodes,
+finishes and frees.
+
+The reference's loop (serve/run.py:238-308) runs either a batch of whole prompts or one token
+for every running request, never both, and reserves prompt + max_new_tokens per request
+against 0.9 of the cache (serve/run.py:273-280).  Differences here:
+
+* a step is mixed: every running request that is decoding gets its one token, and what is left
+  of the step's token budget goes to prompt portions, first come first served;
+* a request finishes in the step that samples its last token, and is freed in that step (the
+  reference decodes a request with max_new_tokens = 1 once more after freeing it,
+  serve/run.py:288,295);
+* what happens when pages run out is decided: with `admission="reserve"` a request is admitted
+  only when pages for prompt + max_new_tokens can be set aside, so a running request never
+  lacks a page; with `admission="optimistic"` pages are taken as requests grow, and when a
+  step does not fit, the most recently admitted running request is preempted: its pages are
+  given back and it returns to the head of the queue to be recomputed from its prompt plus
+  what it has generated (its sampling keys depend only on request and token index, so its
+  tokens do not change).  A request that cannot fit even in an empty cache ends with an error
+  instead of blocking the queue.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, List, Optional, Sequence
+
+from ..config.engine import EngineConfig
+from .batch import Segment
+
+
+@dataclass
+class GenerationRequest:
+    req_id: int
+    prompt: List[int]
+    max_new_tokens: int
+    temperature: float = 0.0
+    keep_logits: bool = False
+    # results
+    generated: List[int] = field(default_factory=list)
+    last_logits: object = None
+    error: Optional[str] = None
+    preemptions: int = 0
+    # progress: tokens of prompt + generated that are in the cache
+    fed: int = 0
+
+    def all_tokens(self) -> List[int]:
+        return self.prompt + self.generated
+
+    def pending(self) -> int:
+        return len(self.prompt) + len(self.generated) - self.fed
+
+    def done(self) -> bool:
+        return len(self.generated) >= self.max_new_tokens
+
+
+@dataclass
+class StepPlan:
+    requests: List[GenerationRequest]
+    counts: List[int]                    # tokens of each request in this step
+    samples: List[bool]                  # whether the step ends the request's pending tokens
+
+
+class Scheduler:
+    """Drives `runner.step` until every request has finished.
+
+    `runner` offers `cache` (a CacheManager), `admit(id) -> bool`, `release(id)` and
+    `step(segments) -> logits`; `sampler.sample(logits, temperatures, request_ids,
+    token_indices) -> tokens`.
+    """
+
+    def __init__(self, runner, sampler, cfg: EngineConfig, eos_token_ids: Optional[Sequence[int]] = None):
+        self.runner, self.sampler, self.cfg = runner, sampler, cfg
+        self.cache = runner.cache
+        self.eos = set(eos_token_ids or ())
+        self.waiting: Deque[GenerationRequest] = deque()
+        self.running: List[GenerationRequest] = []
+        self.finished: List[GenerationRequest] = []
+        self._reserved = [0] * self.cache.num_groups
+        self._reservation = {}
+        self.steps = 0
+        self.step_log: List[dict] = []       # one record per step, for tests and tracing
+
+    # -- life cycle of a request ----------------------------------------------------------------
+    def _total_pages(self, g: int) -> int:
+        return self.cache.pools[g].num_pages
+
+    def _finish(self, r: GenerationRequest, error: Optional[str] = None) -> None:
+        r.error = error
+        if r.req_id in self.cache:
+            self.runner.release(r.req_id)
+        res = self._reservation.pop(r.req_id, None)
+        if res is not None:
+            for g, n in enumerate(res):
+                self._reserved[g] -= n
+        if r in self.running:
+            self.running.remove(r)
+        self.finished.append(r)
+
+    def _preempt(self, r: GenerationRequest) -> None:
+        self.runner.release(r.req_id)
+        self.running.remove(r)
+        r.fed = 0
+        r.preemptions += 1
+        self.waiting.appendleft(r)
+
+    def _try_admit(self, r: GenerationRequest, free: List[int], first_portion: int) -> bool:
+        """Admit the head of the queue if the policy allows it now."""
+        G = self.cache.num_groups
+        if self.cfg.admission == "reserve":
+            need = [self.cache.pages_for_tokens(len(r.prompt) + r.max_new_tokens)] * G
+            if any(self._reserved[g] + need[g] > self._total_pages(g) for g in range(G)):
+                return False
+        else:
+            need = [self.cache.pages_for_tokens(r.fed + first_portion)] * G
+            # keep one spare page per running request, so that a newcomer does not take the page
+            # a decoding request needs at its next page boundary
+            spare = len(self.running)
+            if any(need[g] + spare > free[g] for g in range(G)):
+                return False
+        if not self.runner.admit(r.req_id):
+            return False
+        if self.cfg.admission == "reserve":
+            self._reservation[r.req_id] = need
+            for g in range(G):
+                self._reserved[g] += need[g]
+        self.running.append(r)
+        return True
+
+    def _reject_if_oversize(self, r: GenerationRequest) -> bool:
+        total = len(r.prompt) + r.max_new_tokens
+        if len(r.prompt) == 0:
+            self._finish(r, "empty prompt")
+            return True
+        if total > self.cfg.max_context:
+            self._finish(r, f"prompt ({len(r.prompt)}) + max_new_tokens ({r.max_new_tokens}) exceeds "
+                            f"max_context {self.cfg.max_context}")
+            return True
+        pages = self.cache.pages_for_tokens(total)
+        if any(pages > self._total_pages(g) for g in range(self.cache.num_groups)):
+            self._finish(r, f"the request needs {pages} pages, the cache has "
+                            f"{min(self._total_pages(g) for g in range(self.cache.num_groups))}")
+            return True
+        return False
+
+    # -- planning one step ------------------------------------------------------------------------
+    def plan(self) -> StepPlan:
+        """Choose the requests and token counts of the next step.  May admit and preempt."""
+        cfg = self.cfg
+        G = self.cache.num_groups
+        while True:
+            budget = cfg.max_tokens_per_step
+            free = [self.cache.free_pages(g) for g in range(G)]
+            plan = StepPlan([], [], [])
+            short = None                      # a running request whose portion found no pages
+
+            def try_add(r: GenerationRequest, n: int) -> bool:
+                need = self.cache.pages_needed(r.req_id, r.fed + n)
+                if any(need[g] > free[g] for g in range(G)):
+                    return False
+                for g in range(G):
+                    free[g] -= need[g]
+                plan.requests.append(r)
+                plan.counts.append(n)
+                plan.samples.append(n == r.pending())
+                return True
+
+            # 1. one token for every request that is decoding
+            for r in self.running:
+                if budget == 0:
+                    break
+                if r.pending() == 1:
+                    if try_add(r, 1):
+                        budget -= 1
+                    elif short is None:
+                        short = r
+            # 2. prompt portions of running requests, oldest first
+            for r in self.running:
+                if budget == 0:
+                    break
+                if r.pending() > 1:
+                    n = min(r.pending(), cfg.prefill_chunk, budget)
+                    # a smaller portion may still fit when pages are few
+                    while n > 0 and not try_add(r, n):
+                        n = min(n - 1, (self._fit_tokens(r, free)))
+                    if n > 0:
+                        budget -= n
+                    elif short is None:
+                        short = r
+            if short is not None:
+                # a running request found no page: the youngest gives its pages back, so that
+                # an older request never waits behind a younger one
+                victim = self.running[-1]
+                if len(self.running) == 1:
+                    self._finish(victim, "the cache cannot hold the request's next token")
+                else:
+                    self._preempt(victim)
+                continue
+            # 3. new requests, first come first served, stop at the first that does not fit
+            while self.waiting and budget > 0:
+                r = self.waiting[0]
+                if r.done():
+                    self.waiting.popleft()
+                    self._finish(r)
+                    continue
+                if self._reject_if_oversize(r):
+                    self.waiting.popleft()
+                    continue
+                n = min(r.pending(), cfg.prefill_chunk, budget)
+                if not self._try_admit(r, free, n):
+                    break
+                self.waiting.popleft()
+                if try_add(r, n):
+                    budget -= n
+                else:
+                    # admitted under a reservation but the pages are still held by others
+                    break
+            if plan.requests:
+                return plan
+            if not self.running:
+                if not self.waiting:
+                    return plan
+                # nothing runs and the head of the queue cannot start: it never will
+                r = self.waiting.popleft()
+                self._finish(r, "the request does not fit into the empty cache")
+                continue
+            # running requests exist but the token budget gave none a turn: cannot happen with a
+            # positive budget; stop rather than spin
+            raise RuntimeError("scheduler made no progress")
+
+    def _fit_tokens(self, r: GenerationRequest, free: List[int]) -> int:
+        """Most tokens of r that the free pages can take now."""
+        have = self.cache.tokens_of(r.req_id)
+        room = min(free) * self.cache.page_size + (-have) % self.cache.page_size
+        return room
+
+    # -- running ----------------------------------------------------------------------------------
+    def add(self, requests: Sequence[GenerationRequest]) -> None:
+        self.waiting.extend(requests)
+
+    def step(self) -> bool:
+        """Plan and run one step.  False when nothing is left to do."""
+        plan = self.plan()
+        if not plan.requests:
+            return False
+        segments = []
+        for r, n, s in zip(plan.requests, plan.counts, plan.samples):
+            toks = r.all_tokens()[r.fed: r.fed + n]
+            segments.append(Segment(r.req_id, toks, [n - 1] if s else []))
+        logits = self.runner.step(segments)
+        samplers = [r for r, s in zip(plan.requests, plan.samples) if s]
+        tokens = self.sampler.sample(logits, [r.temperature for r in samplers],
+                                     [r.req_id for r in samplers], [len(r.generated) for r in samplers])
+        self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in plan.requests],
+                                  counts=list(plan.counts), sampled=[r.req_id for r in samplers]))
+        self.steps += 1
+        for r, n in zip(plan.requests, plan.counts):
+            r.fed += n
+        for i, (r, tok) in enumerate(zip(samplers, tokens)):
+            r.generated.append(int(tok))
+            if r.done() or int(tok) in self.eos:
+                if r.keep_logits:
+                    r.last_logits = logits[i].clone()
+                self._finish(r)
+        return True
+
+    def run(self, requests: Sequence[GenerationRequest]) -> List[GenerationRequest]:
+        """Generate for all requests; returns them in the order given."""
+        self.add(requests)
+        while self.step():
+            pass
+        return list(requests)

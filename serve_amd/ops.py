@@ -1,0 +1,235 @@
+"""Python face of the HIP kernels: argument checks on the host, then one C call.
+
+Every function checks on the host that shapes, dtypes, contiguity and device match what the
+kernel and its grid assume, so that a wrong call is an exception and never a wild access on
+the GPU.  There is no CPU path: tensors that are not on a GPU are refused, and a missing
+library that cannot be compiled is an error (`serve_amd.csrc.build.BuildError`).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .csrc.build import load_library
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+c_int = ctypes.c_int
+c_float = ctypes.c_float
+c_void_p = ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype}; the kernels take float32 and bfloat16") from None
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        _check(t.is_cuda, "serve_amd kernels run on the GPU only; got a tensor on " + str(t.device))
+        _check(t.is_contiguous(), "kernel arguments must be contiguous")
+        if dev is None:
+            dev = t.device
+        _check(t.device == dev, "kernel arguments lie on different devices")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ret(code: int, what: str) -> None:
+    if code != 0:
+        reason = {-1: "bad argument", -2: "unsupported combination of dtypes"}.get(code, f"HIP error {code}")
+        raise KernelError(f"{what}: {reason}")
+
+
+def _i32(t: torch.Tensor, n: int, name: str) -> None:
+    _check(t.dtype == torch.int32 and t.numel() >= n, f"{name} must be int32 with at least {n} entries")
+
+
+# ---------------------------------------------------------------------------------------------
+
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[tokens[t]] as fp32.  Token ids must have been checked against the table
+    on the host (the batch builder does)."""
+    _dev(table, tokens, out)
+    T = tokens.numel()
+    _check(table.dim() == 2, "embedding table must be [V, d]")
+    d = table.shape[1]
+    _i32(tokens, T, "tokens")
+    _check(out.dtype == torch.float32 and out.shape == (T, d), "embed output must be fp32 [T, d]")
+    lib = load_library("elementwise")
+    _ret(lib.sa_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out), c_int(T), c_int(d),
+                      _stream()), "embed")
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += delta (fp32 residual stream, in place), out = rmsnorm(x) * weight.
+
+    With `rows`, only the listed rows are produced (out[r] from source row rows[r]) and x is
+    left as it was."""
+    _dev(x, delta, weight, out, rows)
+    _check(x.dtype == torch.float32 and x.dim() == 2, "residual stream must be fp32 [T, d]")
+    T, d = x.shape
+    _check(weight.shape == (d,), f"norm weight must be [{d}]")
+    R = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, R, "rows")
+    _check(out.shape == (R, d), f"norm output must be [{R}, {d}]")
+    if delta is not None:
+        _check(delta.shape == (T, d) and delta.dtype == out.dtype, "delta must be [T, d] in the activation dtype")
+    lib = load_library("elementwise")
+    _ret(lib.sa_add_rmsnorm(_ptr(x), _ptr(delta), _ptr(weight), c_int(_code(weight)), _ptr(out),
+                            c_int(_code(out)), _ptr(rows), c_float(eps), c_int(R), c_int(d), _stream()),
+         "add_rmsnorm")
+    return out
+
+
+def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T with fp32 multiply and accumulate (vector ALU)."""
+    _dev(a, w, out)
+    _check(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm operands must be matrices")
+    M, K = a.shape
+    N = w.shape[0]
+    _check(w.shape[1] == K, f"gemm: inner sizes differ ({K} vs {w.shape[1]})")
+    _check(out.shape == (M, N), f"gemm: output must be [{M}, {N}]")
+    lib = load_library("gemm")
+    _ret(lib.sa_gemm_nt(_ptr(a), c_int(_code(a)), _ptr(w), c_int(_code(w)), _ptr(out), c_int(_code(out)),
+                        c_int(M), c_int(N), c_int(K), _stream()), "gemm_nt")
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+                  slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                  v_pages: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,
+                  rot_dim: int, adjacent_pairs: bool, page_size: int) -> None:
+    """Rotate q (in place) and k; store rotated k and v of every token at its cache slot.
+
+    qkv [T, (Hq + 2 Hk) D]; k_pages [P, Hk, page_size, D]; v_pages [P, Hk, D, page_size];
+    slots[t] = page * page_size + offset.  With `slots=None` only q is rotated (a mixer that
+    reads another layer's cache) and the row holds q alone: qkv is [T, Hq D], Hk = 0."""
+    write = slots is not None
+    _dev(qkv, positions, inv_freq, slots, k_pages, v_pages)
+    T = qkv.shape[0]
+    Hk = num_kv_heads if write else 0
+    _check(qkv.dim() == 2 and qkv.shape[1] == (num_heads + 2 * Hk) * head_dim,
+           f"qkv must be [T, {(num_heads + 2 * Hk) * head_dim}]")
+    _i32(positions, T, "positions")
+    _check(inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dim // 2,
+           f"inv_freq must be fp32 [{rot_dim // 2}]")
+    _check(rot_dim % 2 == 0 and 0 <= rot_dim <= head_dim, "rot_dim must be even and at most head_dim")
+    if write:
+        _i32(slots, T, "slots")
+        P = k_pages.shape[0]
+        _check(k_pages.shape == (P, Hk, page_size, head_dim), "k_pages must be [P, Hk, page_size, D]")
+        _check(v_pages.shape == (P, Hk, head_dim, page_size), "v_pages must be [P, Hk, D, page_size]")
+        _check(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "cache dtype must match activations")
+    lib = load_library("elementwise")
+    _ret(lib.sa_rope_kv_write(_ptr(qkv), c_int(_code(qkv)), _ptr(positions), _ptr(inv_freq), _ptr(slots),
+                              _ptr(k_pages), _ptr(v_pages), c_int(_code(qkv)), c_int(T), c_int(num_heads),
+                              c_int(Hk), c_int(head_dim), c_int(rot_dim), c_int(1 if adjacent_pairs else 0),
+                              c_int(page_size), c_int(1 if write else 0), _stream()), "rope_kv_write")
+
+
+def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
+                           v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
+                           ctx_len: torch.Tensor, seg_of_token: torch.Tensor, num_tokens: int,
+                           num_heads: int, scale: float, window: Optional[int]) -> torch.Tensor:
+    """Attention of every token of the step over its request's cached keys (fp32 arithmetic).
+
+    q is the start of the q block of the fused qkv rows (row stride `q_row_stride` elements)."""
+    _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len, seg_of_token)
+    P, Hk, page_size, D = k_pages.shape
+    _check(v_pages.shape == (P, Hk, D, page_size), "v_pages must be [P, Hk, D, page_size]")
+    _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
+    _check(D <= 256, f"head_dim {D} is above this kernel's limit of 256")
+    T = num_tokens
+    _check(out.shape == (T, num_heads * D) and out.dtype == q.dtype, "attention output must be [T, Hq D]")
+    _check(q.numel() >= (T - 1) * q_row_stride + num_heads * D if T else True, "q is too short")
+    _check(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, "cache dtype must match activations")
+    _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
+    B = block_table.shape[0]
+    _i32(cu_q, B + 1, "cu_q")
+    _i32(ctx_len, B, "ctx_len")
+    _i32(seg_of_token, T, "seg_of_token")
+    lib = load_library("attention_simple")
+    _ret(lib.sa_paged_attention_simple(
+        _ptr(q), c_int(q_row_stride), _ptr(out), c_int(_code(q)), _ptr(k_pages), _ptr(v_pages),
+        c_int(_code(k_pages)), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len),
+        _ptr(seg_of_token), c_int(T), c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size),
+        c_float(scale), c_int(window or 0), _stream()), "paged_attention_simple")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _dev(gate_up, out)
+    T, two_i = gate_up.shape
+    _check(two_i % 2 == 0 and out.shape == (T, two_i // 2) and out.dtype == gate_up.dtype,
+           "silu_mul: out must be [T, I] for gate_up [T, 2 I]")
+    lib = load_library("elementwise")
+    _ret(lib.sa_silu_mul(_ptr(gate_up), _ptr(out), c_int(_code(out)), c_int(T), c_int(two_i // 2), _stream()),
+         "silu_mul")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Optional[torch.Tensor],
+           out: torch.Tensor) -> torch.Tensor:
+    """One token per row of fp32 logits: argmax where temperature is 0 (or None), else the
+    draw argmax(logits / T - log q), q ~ Exp(1) from the row's 64-bit key."""
+    _dev(logits, temperature, keys, out)
+    _check(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be fp32 [R, V]")
+    R, V = logits.shape
+    _i32(out, R, "sample output")
+    if temperature is not None:
+        _check(temperature.dtype == torch.float32 and temperature.numel() == R, "temperature must be fp32 [R]")
+        _check(keys is not None and keys.dtype == torch.int64 and keys.numel() == R, "keys must be int64 [R]")
+    lib = load_library("sampling")
+    _ret(lib.sa_sample(_ptr(logits), _ptr(temperature), _ptr(keys), _ptr(out), c_int(R), c_int(V), _stream()),
+         "sample")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# dispatch between kernels of the same operation
+# ---------------------------------------------------------------------------------------------
+
+def mfma_gemm_available(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """Whether the bf16 MFMA product takes these operands."""
+    return False
+
+
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    raise KernelError("the bf16 MFMA product is not available")
+
+
+def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
+                    v_pages: torch.Tensor, block_table: torch.Tensor, ctx, num_heads: int, scale: float,
+                    window: Optional[int]) -> torch.Tensor:
+    """Attention over the paged cache for all tokens of the step described by `ctx`
+    (`serve_amd.engine.batch.StepContext`)."""
+    return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
+                                  ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

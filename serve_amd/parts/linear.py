@@ -1,0 +1,33 @@
+"""Matrix products of the parts: out = a @ w^T, w stored [out_features, in_features] as the
+reference's nn.Linear weights are (serve/model.py:80-82,95,97,159).
+
+Which kernel runs is decided here and nowhere else:
+
+* float32 activations or weights -> the fp32 vector-ALU product (`ops.gemm_nt`): the true
+  32-bit path, also taken for weights a checkpoint stores in 32-bit;
+* bfloat16 with few rows -> the weight-streaming MFMA kernel (`ops.gemm_bf16_skinny`);
+* bfloat16 with many rows -> the tiled MFMA kernel (`ops.gemm_bf16_tiled`).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import ops
+
+# rows up to which the weight-streaming kernel is used
+SKINNY_MAX_ROWS = 64
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    M = a.shape[0]
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+    if M == 0:
+        return out
+    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and ops.mfma_gemm_available(a, w, out):
+        return ops.gemm_bf16(a, w, out)
+    return ops.gemm_nt(a, w, out)

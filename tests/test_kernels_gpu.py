@@ -1,0 +1,293 @@
+"""Each HIP kernel alone against a plain torch fp32/fp64 reference, at sizes other than the
+engine's: head sizes in steps of 16, odd head counts and groups, widths and vocabularies that
+are no power of two."""
+from __future__ import annotations
+
+import math
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol(dtype):
+    return dict(atol=1e-5, rtol=1e-5) if dtype == "float32" else dict(atol=1e-2, rtol=1e-2)
+
+
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    from serve_amd import ops
+    V, d = 301, 72
+    table = rnd((V, d), DT[dtype], 0)
+    tokens = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
+    out = torch.empty((5, d), dtype=torch.float32, device=DEV)
+    ops.embed(table, tokens, out)
+    torch.testing.assert_close(out, table.float()[tokens.long()], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d,eps", [(72, 1e-5), (2048 + 16, 1e-6)])
+def test_add_rmsnorm(dtype, d, eps):
+    from serve_amd import ops
+    T = 9
+    x = rnd((T, d), torch.float32, 1)
+    x[3] *= 1e-4                                        # a tiny row: eps matters here
+    delta = rnd((T, d), DT[dtype], 2)
+    w = rnd((d,), DT[dtype], 3) * 0.1 + 1
+    x0 = x.clone()
+    y = torch.empty((T, d), dtype=DT[dtype], device=DEV)
+    ops.add_rmsnorm(x, delta, w, eps, y)
+    xs = x0.double() + delta.double()
+    torch.testing.assert_close(x.double(), xs, atol=1e-6, rtol=1e-6)
+    want = xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    torch.testing.assert_close(y.double(), want, **tol(dtype))
+    # without delta, and with a row selection that leaves x alone
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32, device=DEV)
+    x1 = x.clone()
+    y2 = torch.empty((3, d), dtype=DT[dtype], device=DEV)
+    ops.add_rmsnorm(x, delta, w, eps, y2, rows)
+    torch.testing.assert_close(x, x1, atol=0, rtol=0)
+    xs2 = (x1.double() + delta.double())[rows.long()]
+    want2 = xs2 * torch.rsqrt(xs2.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    torch.testing.assert_close(y2.double(), want2, **tol(dtype))
+    y3 = torch.empty((T, d), dtype=DT[dtype], device=DEV)
+    ops.add_rmsnorm(x, None, w, eps, y3)
+    want3 = x1.double() * torch.rsqrt(x1.double().pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    torch.testing.assert_close(y3.double(), want3, **tol(dtype))
+
+
+@pytest.mark.parametrize("a_dt,w_dt,c_dt", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
+                                            ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
+@pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 64, 64), (17, 130, 100), (64, 509, 96), (130, 65, 257)])
+def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
+    from serve_amd import ops
+    a = rnd((M, K), DT[a_dt], 4)
+    w = rnd((N, K), DT[w_dt], 5, 0.1)
+    out = torch.empty((M, N), dtype=DT[c_dt], device=DEV)
+    ops.gemm_nt(a, w, out)
+    want = a.double() @ w.double().T
+    torch.testing.assert_close(out.double(), want, **(tol("float32") if c_dt == "float32" else tol("bfloat16")))
+
+
+# ---------------------------------------------------------------------------------------------
+def rope_ref(x, pos, inv_freq, rot, adjacent):
+    """x [T, H, D] fp64; complex multiply on the rotated part."""
+    T, H, D = x.shape
+    ang = pos.double()[:, None] * inv_freq.double()[None, :]          # [T, rot/2]
+    rotor = torch.polar(torch.ones_like(ang), ang)[:, None, :]
+    xr = x[..., :rot]
+    if adjacent:
+        z = torch.view_as_complex(xr.reshape(T, H, rot // 2, 2).contiguous())
+        o = torch.view_as_real(z * rotor).reshape(T, H, rot)
+    else:
+        z = torch.complex(xr[..., : rot // 2], xr[..., rot // 2:])
+        zz = z * rotor
+        o = torch.cat([zz.real, zz.imag], dim=-1)
+    return torch.cat([o, x[..., rot:]], dim=-1)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("Hq,Hk,D,rot,adjacent,ps", [(4, 2, 16, 16, False, 4), (3, 1, 48, 32, True, 8),
+                                                     (6, 3, 80, 80, False, 16)])
+def test_rope_kv_write(dtype, Hq, Hk, D, rot, adjacent, ps):
+    from serve_amd import ops
+    T, P = 11, 9
+    qkv = rnd((T, (Hq + 2 * Hk) * D), DT[dtype], 6)
+    qkv0 = qkv.clone()
+    pos = torch.tensor([0, 1, 2, 3, 100, 101, 7, 8, 9, 10, 4000], dtype=torch.int32, device=DEV)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    perm = torch.randperm(P * ps, generator=torch.Generator().manual_seed(7))[:T].to(torch.int32).to(DEV)
+    k_pages = torch.zeros((P, Hk, ps, D), dtype=DT[dtype], device=DEV)
+    v_pages = torch.zeros((P, Hk, D, ps), dtype=DT[dtype], device=DEV)
+    ops.rope_kv_write(qkv, pos, inv_freq, perm, k_pages, v_pages, Hq, Hk, D, rot, adjacent, ps)
+    x = qkv0.double().view(T, Hq + 2 * Hk, D)
+    q_want = rope_ref(x[:, :Hq], pos, inv_freq, rot, adjacent)
+    k_want = rope_ref(x[:, Hq:Hq + Hk], pos, inv_freq, rot, adjacent)
+    v_want = x[:, Hq + Hk:]
+    t = dict(atol=2e-4, rtol=1e-5) if dtype == "float32" else tol(dtype)   # angle 4000 rad in fp32
+    torch.testing.assert_close(qkv.double().view(T, -1, D)[:, :Hq], q_want, **t)
+    torch.testing.assert_close(qkv.view(T, -1, D)[:, Hq:], qkv0.view(T, -1, D)[:, Hq:], atol=0, rtol=0)
+    page, off = (perm // ps).long(), (perm % ps).long()
+    torch.testing.assert_close(k_pages.double()[page, :, off, :], k_want, **t)
+    torch.testing.assert_close(v_pages.double()[page, :, :, off], v_want, **t)
+    # every slot that was not addressed is still zero
+    mask = torch.ones((P, ps), dtype=torch.bool, device=DEV)
+    mask[page, off] = False
+    assert k_pages.permute(0, 2, 1, 3)[mask].abs().max().item() == 0
+    assert v_pages.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
+
+
+def test_rope_depends_on_distance_only():
+    """<rope(q, m), rope(k, n)> depends on m - n: shift all positions and compare the scores."""
+    from serve_amd import ops
+    D, H = 32, 2
+    inv_freq = (1.0 / (500000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+    base = rnd((6, 2 * H * D), torch.float32, 8)       # Hq = H, "k" taken from a second call as q
+
+    def scores(shift):
+        x = base.clone()
+        pos = (torch.arange(6, dtype=torch.int32) * 3 + shift).to(DEV)
+        ops.rope_kv_write(x, pos, inv_freq, None, None, None, 2 * H, 0, D, D, False, 1)
+        x = x.view(6, 2 * H, D)
+        return torch.einsum("ihd,jhd->hij", x[:, :H], x[:, H:])
+    torch.testing.assert_close(scores(0), scores(37), atol=2e-5, rtol=1e-5)
+
+
+# ---------------------------------------------------------------------------------------------
+def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False):
+    """segs: list of (ctx_before, q_len).  Builds a paged cache with shuffled pages, runs the
+    kernel, and compares with dense softmax attention per segment."""
+    from serve_amd import ops
+    rng = random.Random(seed)
+    B = len(segs)
+    T = sum(q for _, q in segs)
+    max_ctx = max(c + q for c, q in segs)
+    MP = -(-max_ctx // ps)
+    P = B * MP + 3
+    pages = list(range(P))
+    rng.shuffle(pages)
+    k_pages = rnd((P, Hk, ps, D), DT[dtype], seed + 1)          # unowned pages hold noise
+    v_pages = rnd((P, Hk, D, ps), DT[dtype], seed + 2)
+    bt = torch.zeros((B, MP), dtype=torch.int32)
+    K = [rnd((c + q, Hk, D), DT[dtype], seed + 10 + i) for i, (c, q) in enumerate(segs)]
+    V = [rnd((c + q, Hk, D), DT[dtype], seed + 20 + i) for i, (c, q) in enumerate(segs)]
+    q = rnd((T, Hq * D), DT[dtype], seed + 3)
+    if standout:
+        # one far key per segment gets a score that dominates: scale key 1 and the queries
+        for i in range(B):
+            K[i][1] = K[i][1] * 6
+    for i, (c, ql) in enumerate(segs):
+        n = -(-(c + ql) // ps)
+        for j in range(n):
+            p = pages.pop()
+            bt[i, j] = p
+            lo, hi = j * ps, min((j + 1) * ps, c + ql)
+            k_pages[p, :, : hi - lo, :] = K[i][lo:hi].permute(1, 0, 2)
+            v_pages[p, :, :, : hi - lo] = V[i][lo:hi].permute(1, 2, 0)
+    cu = [0]
+    for _, ql in segs:
+        cu.append(cu[-1] + ql)
+    seg_of = [i for i, (_, ql) in enumerate(segs) for _ in range(ql)]
+    cu_q = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    ctx_len = torch.tensor([c + ql for c, ql in segs], dtype=torch.int32, device=DEV)
+    seg_of_token = torch.tensor(seg_of, dtype=torch.int32, device=DEV)
+    out = torch.empty((T, Hq * D), dtype=DT[dtype], device=DEV)
+    scale = D ** -0.5
+    ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
+                               T, Hq, scale, window)
+    G = Hq // Hk
+    for i, (c, ql) in enumerate(segs):
+        qi = q[cu[i]: cu[i + 1]].double().view(ql, Hq, D)
+        ki = K[i].double().repeat_interleave(G, dim=1)
+        vi = V[i].double().repeat_interleave(G, dim=1)
+        s = torch.einsum("qhd,khd->hqk", qi, ki) * scale
+        qpos = torch.arange(c, c + ql, device=DEV)[:, None]
+        kpos = torch.arange(c + ql, device=DEV)[None, :]
+        vis = kpos <= qpos
+        if window:
+            vis = vis & (qpos - kpos < window)
+        s = s.masked_fill(~vis[None], float("-inf"))
+        want = torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), vi).reshape(ql, Hq * D)
+        torch.testing.assert_close(out[cu[i]: cu[i + 1]].double(), want, **tol(dtype),
+                                   msg=lambda m: f"segment {i} {segs[i]}: {m}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 2, 64, 16), (6, 2, 48, 16),
+                                        (5, 5, 80, 32), (2, 1, 128, 16), (2, 1, 256, 8)])
+def test_paged_attention_simple(dtype, Hq, Hk, D, ps):
+    segs = [(0, 7), (12, 1), (0, 1), (63, 5), (130, 1), (5, 70)]
+    attention_case(dtype, Hq, Hk, D, ps, segs, seed=100 + D)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_paged_attention_simple_window_and_standout(dtype):
+    attention_case(dtype, 4, 2, 32, 8, [(0, 40), (50, 1), (33, 9)], seed=7, window=16)
+    attention_case(dtype, 4, 2, 32, 8, [(0, 300), (299, 1)], seed=8, standout=True)
+
+
+def test_attention_reduces_to_library_routine():
+    """No rotation, no paging subtleties: one request, whole prompt = causal SDPA of the library."""
+    from serve_amd import ops
+    Hq, Hk, D, ps, S = 4, 4, 32, 8, 37
+    q = rnd((S, Hq * D), torch.float32, 1)
+    k = rnd((S, Hk, D), torch.float32, 2)
+    v = rnd((S, Hk, D), torch.float32, 3)
+    P = -(-S // ps)
+    k_pages = torch.zeros((P, Hk, ps, D), device=DEV)
+    v_pages = torch.zeros((P, Hk, D, ps), device=DEV)
+    for j in range(P):
+        lo, hi = j * ps, min(S, (j + 1) * ps)
+        k_pages[j, :, : hi - lo] = k[lo:hi].permute(1, 0, 2)
+        v_pages[j, :, :, : hi - lo] = v[lo:hi].permute(1, 2, 0)
+    bt = torch.arange(P, dtype=torch.int32, device=DEV)[None]
+    out = torch.empty((S, Hq * D), device=DEV)
+    ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt,
+                               torch.tensor([0, S], dtype=torch.int32, device=DEV),
+                               torch.tensor([S], dtype=torch.int32, device=DEV),
+                               torch.zeros(S, dtype=torch.int32, device=DEV), S, Hq, D ** -0.5, None)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.view(S, Hq, D).transpose(0, 1).cpu(), k.transpose(0, 1).cpu(), v.transpose(0, 1).cpu(), is_causal=True)
+    torch.testing.assert_close(out.cpu().view(S, Hq, D), want.transpose(0, 1), atol=1e-5, rtol=1e-5)
+
+
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_silu_mul(dtype):
+    from serve_amd import ops
+    T, I = 5, 333
+    gu = rnd((T, 2 * I), DT[dtype], 9, 3.0)
+    gu[0, :I] = 0                                      # zero gate -> zero
+    out = torch.empty((T, I), dtype=DT[dtype], device=DEV)
+    ops.silu_mul(gu, out)
+    g, u = gu.double()[:, :I], gu.double()[:, I:]
+    torch.testing.assert_close(out.double(), torch.nn.functional.silu(g) * u, **tol(dtype))
+    assert out[0].abs().max().item() == 0
+
+
+def test_sample_greedy_and_ties():
+    from serve_amd import ops
+    R, V = 7, 1000
+    logits = rnd((R, V), torch.float32, 10)
+    logits[2, 400] = logits[2, 900] = 50.0             # tie -> lowest index
+    logits[3, 999] = 60.0                              # last entry
+    logits[4, 0] = 60.0
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(logits, None, None, out)
+    want = torch.argmax(logits, dim=-1)
+    want[2] = 400
+    assert out.tolist() == want.tolist()
+
+
+def test_sample_matches_plain_draw_and_distribution():
+    from serve_amd.sampling.sampler import Sampler
+    from tests.plain import llama_plain
+    V = 16
+    probs = torch.tensor([0.3, 0.2, 0.1, 0.1, 0.05, 0.05, 0.04, 0.04, 0.03, 0.03, 0.02, 0.01, 0.01, 0.01, 0.005, 0.005])
+    probs = probs / probs.sum()
+    logits1 = (probs.log() * 0.8).to(DEV)              # at T = 0.8 the draw follows `probs`
+    sampler = Sampler(seed=123, device=DEV)
+    N = 20000
+    logits = logits1[None].repeat(N, 1).contiguous()
+    toks = sampler.sample(logits, [0.8] * N, [5] * N, list(range(N)))
+    # the same draws from the plain sampler (same noise function), first 200
+    for i in range(200):
+        assert toks[i] == llama_plain.sample(logits1.cpu(), 0.8, seed=123, request_id=5, token_index=i)
+    counts = torch.bincount(torch.tensor(toks), minlength=V).double()
+    chi2 = ((counts - N * probs.double()) ** 2 / (N * probs.double())).sum().item()
+    assert chi2 < 37.7, f"chi-square {chi2:.1f} over 15 degrees of freedom (0.001 quantile 37.7)"
+    # a request's draw does not depend on its row or on the rest of the batch
+    a = sampler.sample(logits[:3].contiguous(), [0.8, 0.8, 0.8], [5, 6, 7], [0, 0, 0])
+    b = sampler.sample(logits[:2].contiguous(), [0.8, 0.0], [7, 5], [0, 0])
+    assert b[0] == a[2] and b[1] == 0

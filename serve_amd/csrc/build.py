@@ -36,9 +36,21 @@ SOURCES: Dict[str, str] = {
     "gemm": "gemm.hip",
     "attention_simple": "attention_simple.hip",
     "sampling": "sampling.hip",
-    "gemm_mfma": "gemm_mfma.hip",
-    "attention_mfma": "attention_mfma.hip",
 }
+
+# variants that are compiled with defines: library name -> list of define sets
+VARIANTS: Dict[str, List[Dict[str, object]]] = {}
+
+
+def all_libraries() -> List[Tuple[str, Optional[Dict[str, object]]]]:
+    """Everything `__graft_entry__.build()` compiles: each library, and each listed variant."""
+    out: List[Tuple[str, Optional[Dict[str, object]]]] = []
+    for name in SOURCES:
+        if name in VARIANTS:
+            out.extend((name, d) for d in VARIANTS[name])
+        else:
+            out.append((name, None))
+    return out
 
 
 class BuildError(RuntimeError):

@@ -77,7 +77,10 @@ def load_weights(model: Model, reader, rt: Runtime) -> None:
     part prepare itself (fused matrices and the like)."""
     present = check_against(model, reader)
     by_owner: Dict[str, Dict[str, torch.Tensor]] = {}
+    tied = bool(model.spec.lm_head.params.get("tied", False))
     for r in present:
+        if r.owner == "lm_head" and tied:
+            continue                    # a tied head uses the embedding table; its own copy is not read
         t = reader.read(r.checkpoint_name)
         t = t.to(device=rt.device, dtype=device_dtype(t.dtype, rt)).contiguous()
         by_owner.setdefault(r.owner, {})[r.local_name] = t

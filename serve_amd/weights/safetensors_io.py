@@ -142,7 +142,7 @@ def write_safetensors(path: str, tensors: Iterable[Tuple[str, torch.Tensor]], me
             if t.dtype not in _NAMES:
                 raise ValueError(f"tensor {name!r}: dtype {t.dtype} cannot be stored")
             t = t.detach().cpu().contiguous()
-            raw = t.view(torch.uint8).numpy().tobytes() if t.numel() else b""
+            raw = t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b""
             header[name] = {"dtype": _NAMES[t.dtype], "shape": list(t.shape),
                             "data_offsets": [offset, offset + len(raw)]}
             data.write(raw)

@@ -1,0 +1,291 @@
+"""The cache manager and the scheduler's decisions, without a GPU: the scheduler drives a fake
+step function whose "logits" are a pure function of each request's token history, so a wrong
+cut, order, position or reuse changes the generated tokens."""
+from __future__ import annotations
+
+import hashlib
+import random
+
+import numpy as np
+import pytest
+
+from serve_amd.cache.manager import FREED, CacheError, CacheManager, PagePool
+from serve_amd.config.engine import EngineConfig
+from serve_amd.engine.batch import OutOfPages, Segment, plan_step
+from serve_amd.engine.scheduler import GenerationRequest, Scheduler
+
+
+# ---------------------------------------------------------------------------------------------
+# cache manager
+# ---------------------------------------------------------------------------------------------
+def test_pool_is_lifo_and_refuses_double_free():
+    p = PagePool(4)
+    a = p.take(3)
+    assert a == [0, 1, 2] and p.take(2) is None and p.num_free == 1
+    p.give_back([1])
+    assert p.take(1) == [1]                       # the page given back last is handed out first
+    with pytest.raises(CacheError):
+        p.give_back([3])                          # never taken
+    p.give_back([0])
+    with pytest.raises(CacheError):
+        p.give_back([0])                          # freed twice
+
+
+def test_ensure_is_all_or_nothing_and_monotone():
+    cm = CacheManager([None], [5], 4, 3, 8)
+    assert cm.admit("a") == 0 and cm.admit("b") == 1
+    assert cm.ensure("a", 9) and cm.block_table("a") == [0, 1, 2]
+    assert cm.ensure("a", 9) and cm.ensure("a", 5) and len(cm.block_table("a")) == 3     # never shrinks
+    before = (cm.free_pages(), list(cm.block_table("b")))
+    assert not cm.ensure("b", 9)                  # needs 3, only 2 free
+    assert (cm.free_pages(), list(cm.block_table("b"))) == before
+    assert cm.ensure("b", 8)
+    cm.check_invariants()
+    assert cm.pages_needed("a", 13) == [1] and cm.pages_needed("new", 13) == [4]
+    cm.release("a")
+    assert cm.free_pages() == 3
+    with pytest.raises(CacheError):
+        cm.release("a")
+    with pytest.raises(CacheError):
+        cm.admit("b")
+    with pytest.raises(CacheError, match="max_context"):
+        cm.ensure("b", 4 * 8 + 1)
+    cm.check_invariants()
+
+
+def test_slots_run_out_and_come_back():
+    cm = CacheManager([None], [8], 4, 2, 4)
+    assert cm.admit(1) is not None and cm.admit(2) is not None and cm.admit(3) is None
+    s = cm.slot_of(1)
+    cm.release(1)
+    assert cm.admit(3) == s
+    cm.check_invariants()
+
+
+def test_windowed_group_gives_pages_back_as_the_window_passes():
+    # group 0 keeps everything, group 1 a window of 6 tokens; page size 4
+    cm = CacheManager([None, 6], [16, 16], 4, 2, 16)
+    cm.admit("r")
+    assert cm.ensure("r", 20)
+    assert len(cm.block_table("r", 0)) == 5 and len(cm.block_table("r", 1)) == 5
+    freed = cm.trim("r", 20)                     # next query is at position >= 20 and sees keys >= 15
+    assert freed == 3                            # pages 0..2 hold keys 0..11, all below 15
+    assert cm.block_table("r", 1)[:3] == [FREED] * 3 and FREED not in cm.block_table("r", 0)
+    assert cm.free_pages(1) == 14 and cm.free_pages(0) == 11
+    assert cm.trim("r", 20) == 0
+    assert cm.ensure("r", 24) and cm.block_table("r", 1)[5] in (0, 1, 2)      # a freed page is used again
+    cm.check_invariants()
+    cm.release("r")
+    assert cm.free_pages(0) == 16 and cm.free_pages(1) == 16
+    cm.check_invariants()
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_orders_lose_nothing(seed):
+    rng = random.Random(seed)
+    cm = CacheManager([None, 5], [23, 11], 4, 6, 10)
+    lengths = {}
+    for step in range(600):
+        live = cm.live_requests()
+        op = rng.random()
+        if op < 0.3 and cm.free_slots():
+            rid = f"r{step}"
+            assert cm.admit(rid) is not None
+            lengths[rid] = 0
+        elif op < 0.8 and live:
+            rid = rng.choice(live)
+            grow = lengths[rid] + rng.randint(1, 9)
+            if grow <= 40:
+                free_before = [cm.free_pages(0), cm.free_pages(1)]
+                if cm.ensure(rid, grow):
+                    lengths[rid] = grow
+                    cm.trim(rid, grow)
+                else:
+                    assert free_before == [cm.free_pages(0), cm.free_pages(1)]
+        elif live:
+            rid = rng.choice(live)
+            cm.release(rid)
+            del lengths[rid]
+        cm.check_invariants()
+        for rid in cm.live_requests():
+            t0 = cm.block_table(rid, 0)
+            assert len(t0) == -(-lengths[rid] // 4) and FREED not in t0
+    for rid in cm.live_requests():
+        cm.release(rid)
+    cm.check_invariants()
+    assert cm.free_pages(0) == 23 and cm.free_pages(1) == 11 and cm.free_slots() == 6
+
+
+def test_plan_step_arrays():
+    cm = CacheManager([None], [10], 4, 4, 8)
+    cm.admit("a")
+    cm.admit("b")
+    lay, host, facts = plan_step([Segment("a", [1, 2, 3, 4, 5], [4]), Segment("b", [7], [0])], cm, 100)
+    v = lambda off, n: host[off: off + n].tolist()   # noqa: E731
+    assert v(lay.token_ids, 6) == [1, 2, 3, 4, 5, 7] and v(lay.positions, 6) == [0, 1, 2, 3, 4, 0]
+    assert v(lay.seg_of_token, 6) == [0, 0, 0, 0, 0, 1] and v(lay.cu_q, 3) == [0, 5, 6]
+    assert v(lay.ctx_len, 2) == [5, 1] and v(lay.logit_rows, 2) == [4, 5]
+    ta, tb = cm.block_table("a"), cm.block_table("b")
+    assert v(lay.slots[0], 6) == [ta[0] * 4, ta[0] * 4 + 1, ta[0] * 4 + 2, ta[0] * 4 + 3, ta[1] * 4, tb[0] * 4]
+    # the next portion continues at position 5, in the middle of a page
+    lay, host, facts = plan_step([Segment("a", [9, 9], [])], cm, 100)
+    assert v(lay.positions, 2) == [5, 6] and v(lay.slots[0], 2) == [ta[1] * 4 + 1, ta[1] * 4 + 2]
+    assert facts["ctx_lens"] == [7] and lay.R == 0
+    # refusals leave everything as it was
+    free = cm.free_pages()
+    with pytest.raises(OutOfPages):
+        plan_step([Segment("a", [1] * 20, []), Segment("b", [1] * 20, [])], cm, 100)
+    assert cm.free_pages() == free and cm.tokens_of("a") == 7
+    with pytest.raises(ValueError, match="vocabulary"):
+        plan_step([Segment("a", [100], [])], cm, 100)
+    with pytest.raises(ValueError, match="twice"):
+        plan_step([Segment("a", [1], []), Segment("a", [1], [])], cm, 100)
+    with pytest.raises(KeyError):
+        plan_step([Segment("zz", [1], [])], cm, 100)
+
+
+# ---------------------------------------------------------------------------------------------
+# scheduler over a fake step function
+# ---------------------------------------------------------------------------------------------
+VOCAB = 97
+
+
+def next_token_of(history):
+    """The fake model: the next token is a hash of the whole history."""
+    h = hashlib.sha256(np.asarray(history, dtype=np.int64).tobytes()).digest()
+    return int.from_bytes(h[:4], "little") % VOCAB
+
+
+class FakeRunner:
+    def __init__(self, num_pages, page_size, max_requests=8, max_context=256):
+        self.cache = CacheManager([None], [num_pages], page_size, max_requests, -(-max_context // page_size))
+        self.history = {}
+        self.steps = []
+
+    def admit(self, rid):
+        if self.cache.admit(rid) is None:
+            return False
+        self.history[rid] = []
+        return True
+
+    def release(self, rid):
+        self.cache.release(rid)
+        del self.history[rid]
+
+    def step(self, segments):
+        lay, host, facts = plan_step(segments, self.cache, VOCAB)      # allocates as the real step does
+        out = []
+        for i, s in enumerate(segments):
+            # positions must continue the request's history
+            assert host[lay.positions + host[lay.cu_q + i]] == len(self.history[s.req_id])
+            for j, t in enumerate(s.tokens):
+                self.history[s.req_id].append(int(t))
+                if j in s.want:
+                    out.append(next_token_of(self.history[s.req_id]))
+        self.steps.append([(s.req_id, len(s.tokens)) for s in segments])
+        self.cache.check_invariants()
+        return out
+
+
+class FakeSampler:
+    def sample(self, logits, temperatures=None, request_ids=None, token_indices=None):
+        return list(logits)
+
+
+def alone(prompt, n):
+    hist, out = list(prompt), []
+    for _ in range(n):
+        t = next_token_of(hist)
+        out.append(t)
+        hist.append(t)
+    return out
+
+
+def make_requests(rng, n, max_prompt=40, max_new=12):
+    return [GenerationRequest(i, [rng.randrange(VOCAB) for _ in range(rng.randint(1, max_prompt))],
+                              rng.randint(1, max_new)) for i in range(n)]
+
+
+@pytest.mark.parametrize("admission", ["reserve", "optimistic"])
+@pytest.mark.parametrize("budget,chunk", [(2048, 2048), (16, 8), (7, 5)])
+def test_every_request_gets_its_own_tokens(admission, budget, chunk):
+    rng = random.Random(1)
+    reqs = make_requests(rng, 12)
+    reqs[3].max_new_tokens = 1                      # the case the reference mishandles (serve/run.py:288,295)
+    runner = FakeRunner(num_pages=64, page_size=4)
+    cfg = EngineConfig(max_tokens_per_step=budget, prefill_chunk=chunk, admission=admission, max_context=256,
+                       page_size=4, num_pages=64)
+    sched = Scheduler(runner, FakeSampler(), cfg)
+    done = sched.run(reqs)
+    for r in done:
+        assert r.error is None and r.generated == alone(r.prompt, r.max_new_tokens), r.req_id
+    assert all(sum(n for _, n in st) <= budget for st in runner.steps)
+    assert all(n <= chunk for st in runner.steps for _, n in st)
+    assert runner.cache.free_pages() == 64 and not runner.cache.live_requests()
+    # first come, first served: requests start in the order given
+    first = {}
+    for i, st in enumerate(runner.steps):
+        for rid, _ in st:
+            first.setdefault(rid, i)
+    assert [first[r.req_id] for r in reqs] == sorted(first[r.req_id] for r in reqs)
+
+
+def test_steps_are_mixed_prompt_portions_ride_with_decodes():
+    rng = random.Random(2)
+    reqs = [GenerationRequest(0, [1] * 5, 10), GenerationRequest(1, [2] * 30, 3)]
+    runner = FakeRunner(num_pages=64, page_size=4)
+    sched = Scheduler(runner, FakeSampler(), EngineConfig(max_tokens_per_step=9, prefill_chunk=8, page_size=4,
+                                                          num_pages=64, max_context=256))
+    sched.run(reqs)
+    assert runner.steps[0] == [(0, 5), (1, 4)]              # budget 9: whole prompt 0, then 4 tokens of prompt 1
+    assert runner.steps[1] == [(0, 1), (1, 8)]              # decode token first, then a portion of prompt 1
+    assert any(len(st) == 2 and st[0][1] == 1 and st[1][1] > 1 for st in runner.steps)
+
+
+def test_reserve_waits_for_pages_and_never_preempts():
+    rng = random.Random(3)
+    reqs = make_requests(rng, 10, max_prompt=20, max_new=10)
+    runner = FakeRunner(num_pages=12, page_size=4)            # 48 tokens: one or two requests at a time
+    sched = Scheduler(runner, FakeSampler(), EngineConfig(admission="reserve", page_size=4, num_pages=12,
+                                                          max_context=48))
+    done = sched.run(reqs)
+    assert all(r.error is None and r.preemptions == 0 and r.generated == alone(r.prompt, r.max_new_tokens)
+               for r in done)
+    assert runner.cache.free_pages() == 12
+
+
+def test_optimistic_preempts_the_youngest_and_tokens_do_not_change():
+    reqs = [GenerationRequest(i, [i + 1] * 10, 14) for i in range(4)]
+    runner = FakeRunner(num_pages=14, page_size=4)            # 56 tokens; the four need 4 * 24 = 96
+    sched = Scheduler(runner, FakeSampler(), EngineConfig(admission="optimistic", page_size=4, num_pages=14,
+                                                          max_context=56))
+    done = sched.run(reqs)
+    assert all(r.error is None and r.generated == alone(r.prompt, r.max_new_tokens) for r in done)
+    assert sum(r.preemptions for r in done) > 0
+    assert done[0].preemptions == 0                           # the oldest request is never the victim
+    assert runner.cache.free_pages() == 14 and not runner.cache.live_requests()
+
+
+@pytest.mark.parametrize("admission", ["reserve", "optimistic"])
+def test_a_request_that_cannot_fit_ends_with_an_error_and_blocks_nobody(admission):
+    reqs = [GenerationRequest(0, [1] * 100, 5), GenerationRequest(1, [2] * 6, 4), GenerationRequest(2, [], 3),
+            GenerationRequest(3, [3] * 6, 0), GenerationRequest(4, [4] * 20, 18)]
+    runner = FakeRunner(num_pages=8, page_size=4, max_context=64)     # 32 tokens in all
+    sched = Scheduler(runner, FakeSampler(), EngineConfig(admission=admission, page_size=4, num_pages=8,
+                                                          max_context=40))
+    done = sched.run(reqs)
+    assert "max_context" in done[0].error and done[0].generated == []
+    assert done[1].error is None and done[1].generated == alone(done[1].prompt, 4)
+    assert done[2].error == "empty prompt"
+    assert done[3].error is None and done[3].generated == []          # nothing asked for
+    assert "pages" in done[4].error                                    # 38 tokens > 32 in the cache
+    assert runner.cache.free_pages() == 8
+
+
+def test_eos_stops_a_request():
+    r = GenerationRequest(0, [5, 6, 7], 50)
+    want = alone(r.prompt, 50)
+    eos = want[4]
+    runner = FakeRunner(num_pages=32, page_size=4)
+    Scheduler(runner, FakeSampler(), EngineConfig(page_size=4, num_pages=32, max_context=128), eos_token_ids=[eos]).run([r])
+    assert r.generated == want[: want.index(eos) + 1]

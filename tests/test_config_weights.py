@@ -1,0 +1,182 @@
+"""Configuration, registry, safetensors reading and writing, weight errors (no GPU)."""
+from __future__ import annotations
+
+import json
+import os
+
+import pytest
+import torch
+
+from serve_amd.config.llama import ConfigError, LlamaConfig
+from serve_amd.models.model import Model
+from serve_amd.parts.base import Runtime
+from serve_amd.registry import get_architecture, known_architectures, load_config
+from serve_amd.weights import loader
+from serve_amd.weights.safetensors_io import CheckpointReader, DictReader, write_safetensors
+from tests import util
+
+
+def hf(**over):
+    d = util.TINY_B.to_hf_dict()
+    d.update(over)
+    return d
+
+
+def test_config_round_trip_and_defaults():
+    for cfg in (util.TINY_A, util.TINY_B, util.TINY_C):
+        assert LlamaConfig.from_hf_dict(cfg.to_hf_dict()) == cfg
+    d = hf()
+    for k in ("num_key_value_heads", "head_dim", "rms_norm_eps", "rope_theta", "rope_scaling", "tie_word_embeddings"):
+        d.pop(k)
+    c = LlamaConfig.from_hf_dict(d)
+    # defaults of the reference's ModelArgs: serve/model.py:29-30; head_dim = dim // n_heads (:91)
+    assert (c.num_key_value_heads, c.head_dim, c.rms_norm_eps, c.rope_theta) == (3, 32, 1e-5, 10000.0)
+    assert c.rope_scaling is None and c.tie_word_embeddings is False
+
+
+def test_head_dim_need_not_be_hidden_over_heads():
+    c = LlamaConfig.from_hf_dict(hf(head_dim=48))
+    spec = get_architecture("LlamaForCausalLM").build_spec(c)
+    shapes = {r.checkpoint_name: r.shape for r in Model(spec).weight_requests()}
+    assert shapes["model.layers.0.self_attn.q_proj.weight"] == (3 * 48, 96)
+    assert shapes["model.layers.0.self_attn.o_proj.weight"] == (96, 3 * 48)
+
+
+@pytest.mark.parametrize("over,word", [
+    (dict(attention_bias=True), "bias"), (dict(mlp_bias=True), "bias"), (dict(hidden_act="gelu"), "hidden_act"),
+    (dict(rope_scaling=dict(rope_type="yarn", factor=2.0)), "rope_type"),
+    (dict(rope_scaling=dict(rope_type="llama3", factor=2.0)), "lacks"),
+    (dict(num_key_value_heads=2), "multiple"), (dict(head_dim=33), "even"), (dict(vocab_size=0), "positive"),
+])
+def test_config_refuses(over, word):
+    with pytest.raises(ConfigError, match=word):
+        LlamaConfig.from_hf_dict(hf(**over))
+
+
+def test_config_missing_keys_are_named():
+    d = hf()
+    d.pop("intermediate_size")
+    d.pop("vocab_size")
+    with pytest.raises(ConfigError, match="intermediate_size") as e:
+        LlamaConfig.from_hf_dict(d)
+    assert "vocab_size" in str(e.value)
+
+
+def test_registry(tmp_path):
+    assert "LlamaForCausalLM" in known_architectures()
+    with pytest.raises(KeyError, match="LlamaForCausalLM"):
+        get_architecture("NopeForCausalLM")
+    folder = util.make_folder(tmp_path, "B")
+    arch, cfg = load_config(folder)
+    assert arch.name == "LlamaForCausalLM" and cfg == util.TINY_B
+    with pytest.raises(FileNotFoundError):
+        load_config(str(tmp_path / "nothing"))
+
+
+def test_spec_is_data():
+    spec = get_architecture("LlamaForCausalLM").build_spec(util.TINY_A)
+    assert [e.layer for e in spec.run_order] == [0, 1] and [e.cache for e in spec.run_order] == [0, 1]
+    assert spec.layers[0].mixer.kind == "gqa_attention" and spec.layers[1].ffn.kind == "swiglu"
+    assert spec.layers[1].mixer.params["position"].params["theta"] == 10000.0
+    m = Model(spec)
+    assert len(m.cache_requests()) == 2 and m.state_requests() == [None, None]
+
+
+def test_safetensors_round_trip_with_the_library(tmp_path):
+    from safetensors.torch import load_file, save_file
+    t = {"a": torch.randn(3, 5).bfloat16(), "b": torch.arange(7, dtype=torch.int64), "c": torch.randn(2, 2, 2),
+         "s": torch.tensor(3.5)}
+    p = str(tmp_path / "x.safetensors")
+    write_safetensors(p, t.items())
+    back = load_file(p)                       # the library reads what we write
+    for k in t:
+        assert back[k].dtype == t[k].dtype and torch.equal(back[k], t[k])
+    p2 = str(tmp_path / "model.safetensors")
+    save_file(t, p2)                          # and we read what the library writes
+    r = CheckpointReader(str(tmp_path))
+    assert sorted(r.names()) == sorted(t)
+    for k in t:
+        dt, shape = r.info(k)
+        assert dt == t[k].dtype and shape == tuple(t[k].shape) and torch.equal(r.read(k), t[k])
+
+
+def test_sharded_folder(tmp_path):
+    a, b = {"x": torch.ones(2)}, {"y": torch.zeros(3)}
+    write_safetensors(str(tmp_path / "m-1.safetensors"), a.items())
+    write_safetensors(str(tmp_path / "m-2.safetensors"), b.items())
+    with open(tmp_path / "model.safetensors.index.json", "w") as f:
+        json.dump({"weight_map": {"x": "m-1.safetensors", "y": "m-2.safetensors"}}, f)
+    r = CheckpointReader(str(tmp_path))
+    assert sorted(r.names()) == ["x", "y"] and torch.equal(r.read("y"), torch.zeros(3))
+    with pytest.raises(FileNotFoundError):
+        CheckpointReader(str(tmp_path / "none"))
+
+
+def test_random_folder_is_a_function_of_seed_and_name(tmp_path):
+    f1 = loader.write_random_model(str(tmp_path / "a"), util.TINY_B, 1)
+    f2 = loader.write_random_model(str(tmp_path / "b"), util.TINY_B, 1)
+    f3 = loader.write_random_model(str(tmp_path / "c"), util.TINY_B, 2)
+    w1, w2, w3 = util.plain_weights(f1), util.plain_weights(f2), util.plain_weights(f3)
+    assert sorted(w1) == sorted(w2) and all(torch.equal(w1[k], w2[k]) for k in w1)
+    assert not torch.equal(w1["model.norm.weight"], w3["model.norm.weight"])
+    assert "lm_head.weight" not in w1                       # tied: no output matrix is written
+    assert "lm_head.weight" in util.plain_weights(util.make_folder(tmp_path, "A"))
+    assert all(v.dtype == torch.bfloat16 for v in w1.values())
+    n = w1["model.norm.weight"].float()
+    e = w1["model.embed_tokens.weight"].float()
+    assert abs(n.mean().item() - 1) < 0.05 and abs(e.std().item() - 0.02) < 0.002
+    assert util.plain_config(f1)["architectures"] == ["LlamaForCausalLM"]
+
+
+def model_of(cfg):
+    return Model(get_architecture("LlamaForCausalLM").build_spec(cfg))
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes():
+    m = model_of(util.TINY_A)
+    t = dict(loader.random_tensors(m, 0))
+    t.pop("model.layers.1.mlp.up_proj.weight")
+    t.pop("model.norm.weight")
+    t["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 63, dtype=torch.bfloat16)
+    t["model.layers.0.self_attn.q_norm.weight"] = torch.zeros(16)
+    t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)      # known and ignored
+    with pytest.raises(loader.WeightError) as e:
+        loader.check_against(m, DictReader(t))
+    err = e.value
+    assert err.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert err.unexpected == ["model.layers.0.self_attn.q_norm.weight"]
+    assert err.wrong_shape == [("model.layers.0.self_attn.q_proj.weight", (64, 63), (64, 64))]
+    text = str(err)
+    for word in ("missing", "unexpected", "wrong shape", "up_proj", "q_norm", "[64, 63]", "[64, 64]"):
+        assert word in text
+
+
+def test_untied_model_without_output_matrix_is_missing_nothing_but_shares_the_table():
+    # a checkpoint without lm_head.weight shares the embedding table, tied flag or not
+    m = model_of(util.TINY_A)
+    t = dict(loader.random_tensors(m, 0))
+    t.pop("lm_head.weight")
+    loader.check_against(m, DictReader(t))
+    # a tied model may still carry the matrix
+    mb = model_of(util.TINY_B)
+    tb = dict(loader.random_tensors(mb, 0))
+    tb["lm_head.weight"] = tb["model.embed_tokens.weight"].clone()
+    loader.check_against(mb, DictReader(tb))
+
+
+def test_dtype_rule():
+    bf, f32 = Runtime.__new__(Runtime), Runtime.__new__(Runtime)
+    bf.dtype, f32.dtype = torch.bfloat16, torch.float32
+    assert loader.device_dtype(torch.bfloat16, bf) == torch.bfloat16
+    assert loader.device_dtype(torch.float16, bf) == torch.bfloat16
+    assert loader.device_dtype(torch.float32, bf) == torch.float32       # stored in 32-bit stays so
+    assert loader.device_dtype(torch.bfloat16, f32) == torch.float32
+    assert loader.device_dtype(torch.int64, bf) == torch.int32 and loader.device_dtype(torch.int16, f32) == torch.int32
+
+
+def test_engine_refuses_to_run_without_a_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is here")
+    from serve_amd.engine.engine import Engine
+    with pytest.raises(RuntimeError, match="GPU"):
+        Engine.from_config(util.TINY_A, 0)

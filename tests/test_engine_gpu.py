@@ -115,7 +115,7 @@ def mixed_trace(rng, vocab, lengths):
 def test_mixed_batches_reuse_pages(tmp_path, name, dtype):
     from serve_amd.engine.batch import Segment
     page_size = 4 if name == "A" else 8
-    lengths = [23, 41, 9, 30, 17, 2, 36, 12]
+    lengths = [23, 41, 9, 30, 17, 2, 36, 12, 40, 28, 33, 5, 19, 38]
     # four live requests of at most 41 tokens: the pool is far smaller than all requests together
     num_pages = 4 * (-(-41 // page_size)) + 1
     folder, engine = engine_for(tmp_path, name, dtype, num_pages=num_pages, page_size=page_size)

@@ -1,0 +1,320 @@
+// Paged attention on the matrix cores, bf16 in, fp32 softmax and accumulation, for prompt
+// portions and single decoded tokens alike.  Compiled once per head size: -DHEAD_DIM=<multiple
+// of 16, at most 128>.
+//
+// Formulas: serve/kernels/attn_prefill.py:56-72,205 and attn_decode.py:99-111,236 (scores scaled
+// by D^-0.5 with log2(e) folded in so that exp2 is used, causal mask by absolute position, online
+// softmax m/l/O, O/l at the end; query head h reads KV head h / G).  Unlike the reference, the
+// key tile (32 keys) is independent of the page size (any multiple of 4), queries of a prompt
+// portion sit at positions ctx_before + j, and long contexts are split over several waves whose
+// partial (m, l, O) are merged with the running maximum (the reference's merge,
+// attn_decode.py:341-348, has none and is switched off).
+//
+// Work item of one wave: (segment, KV head, tile of 16*NT "rows", split of the key range).  The
+// rows of a segment are its (token, query head of the group) pairs, row = token * G + head_in_group,
+// so the G heads that share a KV head share every K and V load.
+//
+// MFMA use (v_mfma_f32_16x16x32_bf16: D[i][j] += sum_k A[i][k] B[k][j]; lane l holds A row l%16,
+// B column l%16, k-slots 8*(l/16)..+7, and D[4*(l/16)+r][l%16]):
+//   S^T = K Q^T : A = 16 keys x 32 dims of K (16-byte loads along D), B = Q^T.  A lane then holds,
+//                 for ITS query column, keys 4g..4g+3 of both 16-key halves: exactly the eight
+//                 k-slots it must supply for the next product, so P never moves between lanes.
+//   O^T = V^T P^T: A = 16 dims x 32 keys of V^T.  Values are stored transposed inside a page
+//                 ([Hk, D, page_size]), so four consecutive keys at one dim are one 8-byte load.
+#include "common.h"
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<head size>"
+#endif
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+union Frag {
+  uint4 u;
+  uint2 h[2];
+  uint16_t s[8];
+  bf16x8_t v;
+};
+
+constexpr int HD = HEAD_DIM;
+constexpr int DC = (HD + 31) / 32;   // 32-wide chunks of the head dim for Q K^T
+constexpr int DT = HD / 16;          // 16-wide tiles of the head dim for P V
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 128, "head size must be a multiple of 16 up to 128");
+
+__device__ __forceinline__ uint32_t pack2bf(float a, float b) {
+  return (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+}
+
+template <int NT>
+__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, float scale_log2e, int window,
+    int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int hk = blockIdx.y;
+  const int seg = blockIdx.z / num_splits;
+  const int sp = blockIdx.z - seg * num_splits;
+  const int G = Hq / Hk;
+
+  const int q_begin = cu_q[seg];
+  const int q_len = cu_q[seg + 1] - q_begin;
+  const int rows_total = q_len * G;
+  const int r0 = tile * (16 * NT);
+  if (r0 >= rows_total) return;
+  const int ctx = ctx_len[seg];
+  const int ctx_before = ctx - q_len;
+  const int j_lo = r0 / G;
+  const int j_hi = min(rows_total - 1, r0 + 16 * NT - 1) / G;
+  const int hi_key = ctx_before + j_hi;
+  int lo_key = 0;
+  if (window > 0) lo_key = max(0, ctx_before + j_lo - window + 1);
+  const int kb_lo = lo_key >> 5;
+  const int kb_hi = hi_key >> 5;
+  const int per = (kb_hi - kb_lo + num_splits) / num_splits;   // ceil((kb_hi - kb_lo + 1) / splits)
+  const int b0 = kb_lo + sp * per;
+  const int b1 = min(kb_hi + 1, b0 + per);
+  const int* bt = block_table + (size_t)seg * max_pages;
+
+  // this lane's query column in each column tile
+  int qpos[NT], tok[NT], head[NT];
+  bool rvalid[NT];
+  Frag qf[NT][DC];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    const int row = r0 + n * 16 + c;
+    rvalid[n] = row < rows_total;
+    const int rowc = min(row, rows_total - 1);
+    const int j = rowc / G;
+    tok[n] = q_begin + j;
+    head[n] = hk * G + (rowc - j * G);
+    qpos[n] = ctx_before + j;
+    const bf16_t* qp = q + (size_t)tok[n] * q_stride + (size_t)head[n] * HD;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      qf[n][dc].u = make_uint4(0, 0, 0, 0);
+      if (dc * 32 + g * 8 < HD) qf[n][dc].u = *reinterpret_cast<const uint4*>(qp + dc * 32 + g * 8);
+    }
+  }
+
+  float m[NT], l[NT];
+  floatx4_t acc[DT][NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    m[n] = -INFINITY;
+    l[n] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt][n] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+  }
+
+  const size_t k_page_stride = (size_t)Hk * page_size * HD;   // elements per page (K and V alike)
+  for (int kb = b0; kb < b1; ++kb) {
+    const int key0 = kb << 5;
+    // every key of the block visible to every row of the tile: no masking needed
+    const bool full = (key0 + 31 <= ctx_before + j_lo) && (window <= 0 || key0 > ctx_before + j_hi - window);
+
+    // ---- S^T = K Q^T --------------------------------------------------------------------
+    floatx4_t s[2][NT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int kk = min(key0 + t * 16 + c, ctx - 1);
+      const int page = max(bt[kk / page_size], 0);
+      const bf16_t* kp = k_pages + (size_t)page * k_page_stride + ((size_t)hk * page_size + kk % page_size) * HD;
+      Frag kf[DC];
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        kf[dc].u = make_uint4(0, 0, 0, 0);
+        if (dc * 32 + g * 8 < HD) kf[dc].u = *reinterpret_cast<const uint4*>(kp + dc * 32 + g * 8);
+      }
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        s[t][n] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc)
+          s[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[dc].v, qf[n][dc].v, s[t][n], 0, 0, 0);
+      }
+    }
+
+    // ---- V^T fragments (issued early so that the loads overlap the softmax) --------------
+    Frag vf[DT];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int run = key0 + h * 16 + 4 * g;                 // first of this lane's 4 keys
+      const int runc = min(run, (ctx - 1) & ~3);
+      const int page = max(bt[runc / page_size], 0);
+      const bf16_t* vp = v_pages + (size_t)page * k_page_stride + (size_t)hk * HD * page_size + runc % page_size;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        vf[dt].h[h] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * page_size);
+      if (!full) {
+        // keys at or beyond the end of the context hold whatever the page held before
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (run + i >= ctx) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vf[dt].s[h * 4 + i] = 0;
+          }
+      }
+    }
+
+    // ---- online softmax over this lane's 8 keys per column, shared across the 4 lane groups
+    Frag pf[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      float v[2][4];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float x = s[t][n][r] * scale_log2e;
+          if (!full) {
+            const int key = key0 + t * 16 + 4 * g + r;
+            const bool vis = key <= qpos[n] && (window <= 0 || key > qpos[n] - window);
+            x = vis ? x : -INFINITY;
+          }
+          v[t][r] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[n], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m[n] - m_safe);
+      m[n] = m_new;
+      float ps = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          v[t][r] = __builtin_amdgcn_exp2f(v[t][r] - m_safe);
+          ps += v[t][r];
+        }
+      l[n] = l[n] * alpha + ps;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[dt][n] *= alpha;
+      pf[n].u = make_uint4(pack2bf(v[0][0], v[0][1]), pack2bf(v[0][2], v[0][3]),
+                           pack2bf(v[1][0], v[1][1]), pack2bf(v[1][2], v[1][3]));
+    }
+
+    // ---- O^T += V^T P^T -------------------------------------------------------------------
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int n = 0; n < NT; ++n)
+        acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
+  }
+
+  // ---- finish ---------------------------------------------------------------------------
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    float lt = l[n];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (!rvalid[n]) continue;
+    if (num_splits == 1) {
+      const float inv = 1.f / lt;
+      bf16_t* op = out + ((size_t)tok[n] * Hq + head[n]) * HD;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        uint2 w;
+        w.x = pack2bf(acc[dt][n][0] * inv, acc[dt][n][1] * inv);
+        w.y = pack2bf(acc[dt][n][2] * inv, acc[dt][n][3] * inv);
+        *reinterpret_cast<uint2*>(op + dt * 16 + 4 * g) = w;
+      }
+    } else {
+      const size_t slot = ((size_t)tok[n] * Hq + head[n]) * num_splits + sp;
+      float* po = part_o + slot * HD;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<float4*>(po + dt * 16 + 4 * g) =
+            make_float4(acc[dt][n][0], acc[dt][n][1], acc[dt][n][2], acc[dt][n][3]);
+      if (g == 0) {
+        part_ml[slot * 2] = m[n];
+        part_ml[slot * 2 + 1] = lt;
+      }
+    }
+  }
+}
+
+// out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s
+__global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o,
+                                                          const float* __restrict__ part_ml,
+                                                          bf16_t* __restrict__ out, int num_splits) {
+  const size_t item = blockIdx.x;                 // token * Hq + head
+  const float* ml = part_ml + item * num_splits * 2;
+  float M = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, ml[2 * s]);
+  float L = 0.f;
+  float o[(HD + 63) / 64];
+#pragma unroll
+  for (int a = 0; a < (HD + 63) / 64; ++a) o[a] = 0.f;
+  for (int s = 0; s < num_splits; ++s) {
+    const float ms = ml[2 * s];
+    if (ms == -INFINITY) continue;                // an empty split
+    const float w = __builtin_amdgcn_exp2f(ms - M);
+    L += ml[2 * s + 1] * w;
+    const float* po = part_o + (item * num_splits + s) * HD;
+#pragma unroll
+    for (int a = 0; a < (HD + 63) / 64; ++a) {
+      const int d = threadIdx.x + a * 64;
+      if (d < HD) o[a] += po[d] * w;
+    }
+  }
+  const float inv = 1.f / L;
+#pragma unroll
+  for (int a = 0; a < (HD + 63) / 64; ++a) {
+    const int d = threadIdx.x + a * 64;
+    if (d < HD) out[item * HD + d] = from_float<bf16_t>(o[a] * inv);
+  }
+}
+
+extern "C" int sa_attention_mfma_head_dim() { return HD; }
+
+// tiles of 16*nt rows per wave: nt = 1 for decode-only steps, NT_PREFILL otherwise
+#if HEAD_DIM <= 64
+#define NT_PREFILL 4
+#else
+#define NT_PREFILL 2
+#endif
+
+extern "C" int sa_attention_mfma_rows_per_tile(int decode_only) { return decode_only ? 16 : 16 * NT_PREFILL; }
+
+extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, const void* k_pages,
+                                       const void* v_pages, const int* block_table, int max_pages,
+                                       const int* cu_q, const int* ctx_len, int B, int T, int max_q_len,
+                                       int Hq, int Hk, int D, int page_size, float scale, int window,
+                                       int num_splits, float* part_o, float* part_ml, hipStream_t stream) {
+  if (T <= 0 || B <= 0) return 0;
+  if (D != HD || Hq <= 0 || Hk <= 0 || Hq % Hk || page_size <= 0 || (page_size & 3) || max_pages <= 0 ||
+      max_q_len <= 0 || num_splits < 1 || (q_stride & 7))
+    return SA_ERR_ARG;
+  if (num_splits > 1 && (!part_o || !part_ml)) return SA_ERR_ARG;
+  if ((long long)B * num_splits > 65535 || Hk > 65535) return SA_ERR_ARG;
+  const int G = Hq / Hk;
+  const bool small = (long long)max_q_len * G <= 16;
+  const int rows_per_tile = small ? 16 : 16 * NT_PREFILL;
+  const int tiles = (int)(((long long)max_q_len * G + rows_per_tile - 1) / rows_per_tile);
+  dim3 grid((tiles + 3) / 4, Hk, B * num_splits), block(256);
+  const float scale_log2e = scale * 1.4426950408889634f;
+#define GO(NT)                                                                                        \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT>), grid, block, 0, stream, (const bf16_t*)q,     \
+                     q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
+                     block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, scale_log2e, window,   \
+                     num_splits, part_o, part_ml)
+  if (small) GO(1);
+  else GO(NT_PREFILL);
+#undef GO
+  SA_LAUNCH_CHECK();
+  if (num_splits > 1) {
+    hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml,
+                       (bf16_t*)out, num_splits);
+    SA_LAUNCH_CHECK();
+  }
+  return 0;
+}

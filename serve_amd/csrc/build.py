@@ -36,10 +36,15 @@ SOURCES: Dict[str, str] = {
     "gemm": "gemm.hip",
     "attention_simple": "attention_simple.hip",
     "sampling": "sampling.hip",
+    "gemm_mfma": "gemm_mfma.hip",
+    "attention_mfma": "attention_mfma.hip",
 }
 
 # variants that are compiled with defines: library name -> list of define sets
-VARIANTS: Dict[str, List[Dict[str, object]]] = {}
+VARIANTS: Dict[str, List[Dict[str, object]]] = {
+    # one library per head size; a model compiles (or finds) only the one it uses
+    "attention_mfma": [{"HEAD_DIM": d} for d in range(16, 129, 16)],
+}
 
 
 def all_libraries() -> List[Tuple[str, Optional[Dict[str, object]]]]:

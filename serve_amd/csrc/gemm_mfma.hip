@@ -1,0 +1,200 @@
+// bf16 matrix products on the matrix cores for few rows of activations (decode steps and short
+// prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
+//
+// The work is bound by reading W.  A wave owns RT tiles of 16 rows of W and walks a slice of K in
+// steps of 32; the KS waves of a workgroup split K between them and add their partial sums
+// through LDS, so no atomics and a fixed summation order.  The MFMA computes the transposed
+// tile: operand "A" of v_mfma_f32_16x16x32_bf16 is a 16x32 tile of W (lane l: row l%16, k-slots
+// 8*(l/16)..+7), operand "B" is 32x16 of activations (lane l: activation row l%16, same k-slots),
+// and the result gives lane l the four consecutive outputs C[m = l%16][n = 4*(l/16) .. +3],
+// which are contiguous in C.
+//
+// The SWIGLU variant reads gate rows n and up rows I + n of the stacked matrix in the same wave
+// and stores silu(gate) * up (serve/model.py:85), so the [M, 2I] intermediate never exists.
+//
+// Requirements, checked by the caller: K % 8 == 0 (16-byte rows), pointers 16-byte aligned.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+union Frag {
+  uint4 u;
+  bf16x8_t v;
+};
+
+#define KU 4  // k-chunks of 32 loaded before their products are issued
+
+template <int RT, int MT, int KS, typename TC, bool SWIGLU>
+__global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
+                                                             const bf16_t* __restrict__ W,
+                                                             TC* __restrict__ C, int M, int N, int K,
+                                                             int up_offset) {
+  static_assert(KS * RT * MT <= 64, "partial sums must fit into 64 KB of LDS");
+  static_assert(!SWIGLU || RT == 2, "the SwiGLU variant pairs one gate tile with one up tile");
+  __shared__ float red[KS][RT * MT * 4][64];
+
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int n0 = blockIdx.x * (SWIGLU ? 16 : RT * 16);
+  const int m0 = blockIdx.y * (MT * 16);
+
+  const int nchunks = (K + 31) >> 5;
+  const int per = (nchunks + KS - 1) / KS;
+  const int ch_begin = wave * per;
+  const int ch_end = min(nchunks, ch_begin + per);
+
+  const bf16_t* wrow[RT];
+  bool wok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    int n;
+    if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
+    else n = n0 + rt * 16 + c;
+    wok[rt] = SWIGLU ? (n0 + c < N) : (n < N);
+    wrow[rt] = W + (size_t)(wok[rt] ? n : 0) * K;
+  }
+  const bf16_t* arow[MT];
+  bool aok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + mt * 16 + c;
+    aok[mt] = m < M;
+    arow[mt] = A + (size_t)(aok[mt] ? m : 0) * K;
+  }
+
+  floatx4_t acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int ch = ch_begin; ch < ch_end; ch += KU) {
+    Frag wf[RT][KU], af[MT][KU];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int k = (ch + u) * 32 + g * 8;
+      const bool kin = (ch + u) < ch_end && k < K;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        wf[rt][u].u = zero;
+        if (kin && wok[rt]) wf[rt][u].u = *reinterpret_cast<const uint4*>(wrow[rt] + k);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        af[mt][u].u = zero;
+        if (kin && aok[mt]) af[mt][u].u = *reinterpret_cast<const uint4*>(arow[mt] + k);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < KU; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][u].v, af[mt][u].v, acc[rt][mt], 0, 0, 0);
+  }
+
+  // add the KS partial sums in a fixed order: every wave stores, wave 0 sums and writes
+  if (KS > 1) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][(rt * MT + mt) * 4 + r][lane] = acc[rt][mt][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float s = acc[rt][mt][r];
+          for (int w = 1; w < KS; ++w) s += red[w][(rt * MT + mt) * 4 + r][lane];
+          acc[rt][mt][r] = s;
+        }
+  }
+
+  const int ldc = N;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + mt * 16 + c;
+    if (m >= M) continue;
+    if (SWIGLU) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = n0 + 4 * g + r;
+        if (n < N) {
+          const float gt = acc[0][mt][r];
+          const float up = acc[1][mt][r];
+          C[(size_t)m * ldc + n] = from_float<TC>((gt / (1.f + __expf(-gt))) * up);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = n0 + rt * 16 + 4 * g + r;
+          if (n < N) C[(size_t)m * ldc + n] = from_float<TC>(acc[rt][mt][r]);
+        }
+    }
+  }
+}
+
+template <int RT, int MT, int KS, typename TC, bool SWIGLU>
+static int launch_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
+                         hipStream_t stream) {
+  dim3 grid((N + (SWIGLU ? 16 : RT * 16) - 1) / (SWIGLU ? 16 : RT * 16), (M + MT * 16 - 1) / (MT * 16));
+  if (grid.y > 65535) return SA_ERR_ARG;
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, MT, KS, TC, SWIGLU>), grid, dim3(64 * KS), 0, stream,
+                     (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, up_offset);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename TC, bool SWIGLU>
+static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
+                       hipStream_t stream) {
+  // rows of activations per workgroup: 16, 32 or 64 (larger M loops over grid.y)
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  // many weight rows: 2 row tiles per wave and 4 waves; few rows: 1 tile and 16 waves splitting K
+  const bool wide = SWIGLU || N >= 8192;
+#define GO(RT, MT, KS) return launch_skinny<RT, MT, KS, TC, SWIGLU>(A, W, C, M, N, K, up_offset, stream)
+  if (wide) {
+    if (mt == 1) GO(2, 1, 4);
+    if (mt == 2) GO(2, 2, 4);
+    GO(2, 4, 4);
+  }
+  if constexpr (!SWIGLU) {
+    // 16 waves leave 128 registers a lane, enough only for one activation tile
+    if (mt == 1) GO(1, 1, 16);
+    if (mt == 2) GO(1, 2, 8);
+    GO(1, 4, 8);
+  }
+#undef GO
+  return SA_ERR_ARG;
+}
+
+// C = A W^T; c_dtype SA_BF16 or SA_F32
+extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K,
+                                   hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K & 7)) return SA_ERR_ARG;
+  if (c_dtype == SA_BF16) return pick_skinny<bf16_t, false>(A, W, C, M, N, K, 0, stream);
+  if (c_dtype == SA_F32) return pick_skinny<float, false>(A, W, C, M, N, K, 0, stream);
+  return SA_ERR_UNSUPPORTED;
+}
+
+// C[M, I] = silu(A Wg^T) * (A Wu^T) with W = [Wg; Wu] stacked as [2 I, K]
+extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C, int M, int I, int K,
+                                          hipStream_t stream) {
+  if (M <= 0 || I <= 0) return 0;
+  if (K <= 0 || (K & 7)) return SA_ERR_ARG;
+  return pick_skinny<bf16_t, true>(A, W, C, M, I, K, I, stream);
+}

@@ -214,22 +214,127 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Opti
 
 
 # ---------------------------------------------------------------------------------------------
-# dispatch between kernels of the same operation
+# bf16 matrix-core kernels
 # ---------------------------------------------------------------------------------------------
+SKINNY_MAX_ROWS = 64          # above this the weights would be streamed more than once per product
+
+
+def _aligned16(*tensors: torch.Tensor) -> bool:
+    return all(t.data_ptr() % 16 == 0 for t in tensors)
+
 
 def mfma_gemm_available(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
-    """Whether the bf16 MFMA product takes these operands."""
-    return False
+    """Whether the bf16 matrix-core products take these operands: bf16 in, bf16 or fp32 out,
+    inner size a multiple of 8 (16-byte rows)."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and out.dtype in (torch.bfloat16, torch.float32) and a.shape[1] % 8 == 0 and _aligned16(a, w, out))
+
+
+def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = a @ w^T on the matrix cores, weights streamed once per 64 rows of a."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _check(w.shape == (N, K) and out.shape == (M, N), "gemm_bf16_skinny: shapes do not match")
+    _check(mfma_gemm_available(a, w, out), "gemm_bf16_skinny needs bf16 operands, K % 8 == 0 and 16-byte alignment")
+    lib = load_library("gemm_mfma")
+    _ret(lib.sa_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), c_int(_code(out)), c_int(M), c_int(N), c_int(K),
+                                 _stream()), "gemm_bf16_skinny")
+    return out
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    raise KernelError("the bf16 MFMA product is not available")
+    """bf16 product: the weight-streaming kernel for few rows, the BLAS library for many (the
+    reference leaves all of its products to the library, serve/model.py:80-82,95,97,159).  The
+    library writes bf16; fp32 output always takes the kernel."""
+    if a.shape[0] <= SKINNY_MAX_ROWS or out.dtype != torch.bfloat16:
+        return gemm_bf16_skinny(a, w, out)
+    _dev(a, w, out)
+    torch.mm(a, w.t(), out=out)
+    return out
 
+
+def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) for w_gate_up = [Wg; Wu] ([2 I, K]), one kernel."""
+    _dev(a, w_gate_up, out)
+    M, K = a.shape
+    I = w_gate_up.shape[0] // 2
+    _check(w_gate_up.shape == (2 * I, K) and out.shape == (M, I), "swiglu_bf16: shapes do not match")
+    _check(a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+           and K % 8 == 0 and _aligned16(a, w_gate_up, out), "swiglu_bf16 needs bf16 operands and K % 8 == 0")
+    lib = load_library("gemm_mfma")
+    _ret(lib.sa_gemm_bf16_skinny_swiglu(_ptr(a), _ptr(w_gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
+                                        _stream()), "swiglu_bf16")
+    return out
+
+
+MFMA_ATTENTION_HEAD_DIMS = tuple(range(16, 129, 16))
+
+
+def mfma_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_stride: int) -> bool:
+    P, Hk, page_size, D = k_pages.shape
+    return (q.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and D in MFMA_ATTENTION_HEAD_DIMS
+            and page_size % 4 == 0 and q_row_stride % 8 == 0 and q.data_ptr() % 16 == 0)
+
+
+def attention_splits(decode_only: bool, num_segments: int, num_kv_heads: int, max_ctx_len: int) -> int:
+    """Into how many parts the key range of a decode step is cut so that the chip is filled:
+    about 2048 waves in all, and no part shorter than 128 keys."""
+    if not decode_only:
+        return 1
+    by_length = max(1, max_ctx_len // 128)
+    by_waves = max(1, 2048 // max(1, num_segments * num_kv_heads))
+    return max(1, min(by_length, by_waves, 64))
+
+
+def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
+                         v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
+                         ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int, scale: float,
+                         window: Optional[int], num_splits: int = 1) -> torch.Tensor:
+    """bf16 attention on the matrix cores (head sizes 16..128 in steps of 16, page sizes that are
+    multiples of 4)."""
+    _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
+    P, Hk, page_size, D = k_pages.shape
+    _check(mfma_attention_available(q, k_pages, q_row_stride),
+           f"paged_attention_mfma takes bf16, head sizes {MFMA_ATTENTION_HEAD_DIMS} and page sizes that are "
+           f"multiples of 4; got head size {D}, page size {page_size}")
+    _check(v_pages.shape == (P, Hk, D, page_size) and v_pages.dtype == torch.bfloat16,
+           "v_pages must be bf16 [P, Hk, D, page_size]")
+    _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
+    T = num_tokens
+    _check(out.shape == (T, num_heads * D) and out.dtype == torch.bfloat16, "attention output must be bf16 [T, Hq D]")
+    _check(q.numel() >= (T - 1) * q_row_stride + num_heads * D if T else True, "q is too short")
+    _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
+    B = block_table.shape[0]
+    _i32(cu_q, B + 1, "cu_q")
+    _i32(ctx_len, B, "ctx_len")
+    _check(1 <= max_q_len <= max(T, 1) and num_splits >= 1, "max_q_len / num_splits out of range")
+    part_o = part_ml = None
+    if num_splits > 1:
+        part_o = torch.empty((T * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
+    lib = load_library("attention_mfma", {"HEAD_DIM": D})
+    _ret(lib.sa_paged_attention_mfma(
+        _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(T), c_int(max_q_len),
+        c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0),
+        c_int(num_splits), _ptr(part_o), _ptr(part_ml), _stream()), "paged_attention_mfma")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# dispatch between kernels of the same operation
+# ---------------------------------------------------------------------------------------------
 
 def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                     v_pages: torch.Tensor, block_table: torch.Tensor, ctx, num_heads: int, scale: float,
                     window: Optional[int]) -> torch.Tensor:
     """Attention over the paged cache for all tokens of the step described by `ctx`
-    (`serve_amd.engine.batch.StepContext`)."""
+    (`serve_amd.engine.batch.StepContext`): the matrix-core kernel for bf16 where it takes the
+    sizes, else the general fp32-arithmetic kernel."""
+    if mfma_attention_available(q, k_pages, q_row_stride):
+        splits = attention_splits(ctx.decode_only, ctx.num_segments, k_pages.shape[1], ctx.max_ctx_len)
+        return paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
+                                    ctx.num_tokens, ctx.max_q_len, num_heads, scale, window, splits)
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                   ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

@@ -6,7 +6,7 @@ Which kernel runs is decided here and nowhere else:
 * float32 activations or weights -> the fp32 vector-ALU product (`ops.gemm_nt`): the true
   32-bit path, also taken for weights a checkpoint stores in 32-bit;
 * bfloat16 with few rows -> the weight-streaming MFMA kernel (`ops.gemm_bf16_skinny`);
-* bfloat16 with many rows -> the tiled MFMA kernel (`ops.gemm_bf16_tiled`).
+* bfloat16 with many rows -> the BLAS library, as the reference does for all of its products.
 """
 from __future__ import annotations
 
@@ -15,9 +15,6 @@ from typing import Optional
 import torch
 
 from .. import ops
-
-# rows up to which the weight-streaming kernel is used
-SKINNY_MAX_ROWS = 64
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -28,6 +25,6 @@ def linear(a: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
     if M == 0:
         return out
-    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and ops.mfma_gemm_available(a, w, out):
+    if ops.mfma_gemm_available(a, w, out):
         return ops.gemm_bf16(a, w, out)
     return ops.gemm_nt(a, w, out)

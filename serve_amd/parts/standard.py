@@ -172,9 +172,13 @@ class SwiGLU(Part):
         self.w_down = tensors["down_proj.weight"]
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        gu = linear(h, self.w_gate_up)
         a = self.rt.empty((h.shape[0], self.intermediate_size))
-        ops.silu_mul(gu, a)
+        if (h.shape[0] <= ops.SKINNY_MAX_ROWS and h.dtype == torch.bfloat16
+                and self.w_gate_up.dtype == torch.bfloat16 and self.hidden_size % 8 == 0):
+            ops.swiglu_bf16(h, self.w_gate_up, a)          # product and gate in one kernel
+        else:
+            gu = linear(h, self.w_gate_up)
+            ops.silu_mul(gu, a)
         return linear(a, self.w_down)
 
 

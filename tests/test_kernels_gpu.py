@@ -146,7 +146,7 @@ def test_rope_depends_on_distance_only():
 
 
 # ---------------------------------------------------------------------------------------------
-def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False):
+def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False, kernel="simple", splits=1):
     """segs: list of (ctx_before, q_len).  Builds a paged cache with shuffled pages, runs the
     kernel, and compares with dense softmax attention per segment."""
     from serve_amd import ops
@@ -185,8 +185,12 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     seg_of_token = torch.tensor(seg_of, dtype=torch.int32, device=DEV)
     out = torch.empty((T, Hq * D), dtype=DT[dtype], device=DEV)
     scale = D ** -0.5
-    ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
-                               T, Hq, scale, window)
+    if kernel == "simple":
+        ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
+                                   T, Hq, scale, window)
+    else:
+        ops.paged_attention_mfma(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
+                                 max(ql for _, ql in segs), Hq, scale, window, splits)
     G = Hq // Hk
     for i, (c, ql) in enumerate(segs):
         qi = q[cu[i]: cu[i + 1]].double().view(ql, Hq, D)
@@ -292,3 +296,114 @@ def test_sample_matches_plain_draw_and_distribution():
     a = sampler.sample(logits[:3].contiguous(), [0.8, 0.8, 0.8], [5, 6, 7], [0, 0, 0])
     b = sampler.sample(logits[:2].contiguous(), [0.8, 0.0], [7, 5], [0, 0])
     assert b[0] == a[2] and b[1] == 0
+
+
+# ---------------------------------------------------------------------------------------------
+# bf16 matrix-core kernels
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 2, 64, 16), (6, 2, 48, 16),
+                                        (5, 5, 80, 32), (2, 1, 128, 16), (32, 8, 64, 16), (24, 8, 128, 16),
+                                        (20, 1, 64, 8), (7, 7, 96, 4), (3, 3, 112, 12)])
+def test_paged_attention_mfma_mixed(Hq, Hk, D, ps):
+    segs = [(0, 7), (12, 1), (0, 1), (63, 5), (130, 1), (5, 70), (31, 2), (0, 33)]
+    attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=200 + D, kernel="mfma")
+
+
+@pytest.mark.parametrize("Hq,Hk,D,ps,splits", [(4, 2, 16, 4, 3), (8, 2, 64, 16, 4), (32, 8, 64, 16, 7),
+                                               (24, 8, 128, 16, 2), (3, 1, 32, 8, 64)])
+def test_paged_attention_mfma_decode_with_splits(Hq, Hk, D, ps, splits):
+    segs = [(12, 1), (0, 1), (130, 1), (517, 1), (31, 1), (32, 1), (63, 1), (64, 1)]
+    attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=300 + D, kernel="mfma", splits=splits)
+
+
+def test_paged_attention_mfma_window_standout_and_long_prompt():
+    attention_case("bfloat16", 4, 2, 32, 8, [(0, 40), (50, 1), (33, 9), (100, 3)], seed=7, window=16, kernel="mfma")
+    attention_case("bfloat16", 4, 2, 32, 8, [(90, 1), (200, 1)], seed=9, window=48, kernel="mfma", splits=3)
+    attention_case("bfloat16", 4, 2, 64, 16, [(0, 300), (299, 1)], seed=8, standout=True, kernel="mfma")
+    attention_case("bfloat16", 8, 2, 64, 16, [(0, 700)], seed=10, kernel="mfma")
+
+
+def test_paged_attention_mfma_ignores_what_lies_beyond_the_context():
+    """Slots of the last page beyond the context and unowned pages may hold anything, NaN
+    included: p = 0 must not meet a NaN in the product."""
+    from serve_amd import ops
+    Hq, Hk, D, ps = 4, 2, 64, 16
+    for ctx in (1, 5, 16, 17, 37):
+        P = 6
+        k_pages = torch.full((P, Hk, ps, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+        v_pages = torch.full((P, Hk, D, ps), float("nan"), dtype=torch.bfloat16, device=DEV)
+        K, V = rnd((ctx, Hk, D), torch.bfloat16, 1), rnd((ctx, Hk, D), torch.bfloat16, 2)
+        bt = torch.tensor([[4, 1, 3]], dtype=torch.int32, device=DEV)
+        for j in range(-(-ctx // ps)):
+            lo, hi = j * ps, min(ctx, (j + 1) * ps)
+            k_pages[bt[0, j], :, : hi - lo] = K[lo:hi].permute(1, 0, 2)
+            v_pages[bt[0, j], :, :, : hi - lo] = V[lo:hi].permute(1, 2, 0)
+        q = rnd((1, Hq * D), torch.bfloat16, 3)
+        out = torch.empty((1, Hq * D), dtype=torch.bfloat16, device=DEV)
+        for splits in (1, 2):
+            ops.paged_attention_mfma(q, Hq * D, out, k_pages, v_pages, bt,
+                                     torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+                                     torch.tensor([ctx], dtype=torch.int32, device=DEV), 1, 1, Hq, D ** -0.5, None, splits)
+            s = torch.einsum("hd,khd->hk", q.double().view(Hq, D), K.double().repeat_interleave(2, 1)) * D ** -0.5
+            want = torch.einsum("hk,khd->hd", torch.softmax(s, -1), V.double().repeat_interleave(2, 1)).reshape(1, -1)
+            torch.testing.assert_close(out.double(), want, **tol("bfloat16"))
+
+
+@pytest.mark.parametrize("c_dt", ["bfloat16", "float32"])
+@pytest.mark.parametrize("M,N,K", [(1, 70, 40), (3, 64, 64), (8, 3072, 2048), (16, 509, 96), (17, 130, 104),
+                                   (33, 2048, 8192), (64, 8200, 256), (100, 77, 1024), (8, 128256 // 8, 192)])
+def test_gemm_bf16_skinny(c_dt, M, N, K):
+    from serve_amd import ops
+    a = rnd((M, K), torch.bfloat16, 4)
+    w = rnd((N, K), torch.bfloat16, 5, 0.05)
+    out = torch.empty((M, N), dtype=DT[c_dt], device=DEV)
+    ops.gemm_bf16_skinny(a, w, out)
+    want = a.double() @ w.double().T
+    t = dict(atol=2e-4 * K ** 0.5, rtol=1e-4) if c_dt == "float32" else dict(atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(out.double(), want, **t)
+    # the large-matrix route gives the same numbers up to bf16 rounding
+    if c_dt == "bfloat16":
+        out2 = torch.empty_like(out)
+        ops.gemm_bf16(a, w, out2)
+        torch.testing.assert_close(out2.double(), want, atol=2e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 192, 64), (8, 8192, 2048), (20, 320, 192), (64, 1000, 96)])
+def test_swiglu_bf16(M, I, K):
+    from serve_amd import ops
+    a = rnd((M, K), torch.bfloat16, 6)
+    w = rnd((2 * I, K), torch.bfloat16, 7, 0.1)
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=DEV)
+    ops.swiglu_bf16(a, w, out)
+    gu = a.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+    torch.testing.assert_close(out.double(), want, atol=2e-2, rtol=1e-2)
+    # the unfused route agrees
+    gu_b = torch.empty((M, 2 * I), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_skinny(a, w, gu_b)
+    out2 = torch.empty_like(out)
+    ops.silu_mul(gu_b, out2)
+    torch.testing.assert_close(out2.double(), want, atol=3e-2, rtol=2e-2)
+
+
+def test_kernels_refuse_what_they_do_not_take():
+    from serve_amd import ops
+    a = rnd((4, 12), torch.bfloat16, 1)
+    w = rnd((8, 12), torch.bfloat16, 2)
+    out = torch.empty((4, 8), dtype=torch.bfloat16, device=DEV)
+    assert not ops.mfma_gemm_available(a, w, out)               # K = 12 is no multiple of 8
+    with pytest.raises(ops.KernelError):
+        ops.gemm_bf16_skinny(a, w, out)
+    ops.gemm_nt(a, w, out)                                      # the general product takes it
+    with pytest.raises(ops.KernelError, match="GPU only"):
+        ops.gemm_nt(a.cpu(), w.cpu(), out.cpu())
+    k_pages = torch.zeros((2, 1, 8, 144), dtype=torch.bfloat16, device=DEV)
+    assert not ops.mfma_attention_available(rnd((1, 144), torch.bfloat16, 1), k_pages, 144)   # head size 144
+    with pytest.raises(ops.KernelError, match="256"):
+        big = torch.zeros((2, 1, 8, 272), dtype=torch.float32, device=DEV)
+        ops.paged_attention_simple(rnd((1, 272), torch.float32, 1), 272, torch.empty((1, 272), device=DEV), big,
+                                   torch.zeros((2, 1, 272, 8), device=DEV),
+                                   torch.zeros((1, 1), dtype=torch.int32, device=DEV),
+                                   torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+                                   torch.tensor([1], dtype=torch.int32, device=DEV),
+                                   torch.zeros(1, dtype=torch.int32, device=DEV), 1, 1, 1.0, None)

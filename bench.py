@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Benchmark of the engine on one MI355X: decoded tokens per second of a Llama-3.2-1B-shaped
+model with random weights, at batch 8 and a context of 4,096 tokens, page size 16, bfloat16.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the whole batch (scheduler, step function from its HIP graph,
+sampling, tokens back on the host).  One JSON line is printed; beside the main value it holds
+the prefill rate of one 2,048-token prompt with its fraction of the bf16 matrix peak, the
+decode step's fraction of the HBM peak, and decode rates at batch 1 and 64 on 256-token
+prompts with 256 generated tokens (the workload of the reference's benchmark script,
+serve/benchmark.py:43-46, with fixed instead of uniform lengths).  The reference publishes no
+number for this model, so `vs_baseline` is null.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12            # bytes/s, MI355X
+BF16_PEAK = 2.5e15           # dense bf16 MFMA flop/s, MI355X
+
+
+def model_config(layers: int):
+    from serve_amd.config.llama import Llama3RopeScaling, LlamaConfig
+    return LlamaConfig(vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_hidden_layers=layers,
+                       num_attention_heads=32, num_key_value_heads=8, head_dim=64, rms_norm_eps=1e-5,
+                       rope_theta=500000.0,
+                       rope_scaling=Llama3RopeScaling(32.0, 1.0, 4.0, 8192), tie_word_embeddings=True)
+
+
+def weight_bytes(cfg) -> int:
+    d, D = cfg.hidden_size, cfg.head_dim
+    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D * d + d * cfg.num_attention_heads * D
+                 + 3 * d * cfg.intermediate_size + 2 * d)
+    return 2 * (per_layer * cfg.num_hidden_layers + cfg.vocab_size * d + d)
+
+
+def kv_bytes_per_token(cfg) -> int:
+    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * 2
+
+
+def prefill_flops(cfg, T: int) -> float:
+    d, D = cfg.hidden_size, cfg.head_dim
+    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D * d + d * cfg.num_attention_heads * D
+                 + 3 * d * cfg.intermediate_size)
+    matmul = 2.0 * per_layer * cfg.num_hidden_layers * T + 2.0 * cfg.vocab_size * d
+    attention = 4.0 * cfg.num_attention_heads * D * cfg.num_hidden_layers * (T * (T + 1) / 2)
+    return matmul + attention
+
+
+def random_prompts(n: int, length: int, vocab: int, seed: int):
+    import random
+    rng = random.Random(seed)
+    return [[rng.randrange(vocab) for _ in range(length)] for _ in range(n)]
+
+
+def decode_run(engine, batch: int, prompt_len: int, warmup: int, steps: int, seed: int):
+    """Prefill `batch` prompts, run `warmup` untimed and `steps` timed decode steps.
+    Returns (seconds, mean context during the timed steps)."""
+    import torch
+    from serve_amd.engine.scheduler import GenerationRequest, Scheduler
+    prompts = random_prompts(batch, prompt_len, engine.model.spec.vocab_size, seed)
+    reqs = [GenerationRequest(i, p, warmup + steps + 2) for i, p in enumerate(prompts)]
+    sched = Scheduler(engine.runner, engine.sampler, engine.cfg)
+    sched.add(reqs)
+    while any(r.pending() > 1 or r.fed == 0 for r in reqs):
+        assert sched.step()
+    for _ in range(warmup):
+        assert sched.step()
+    torch.cuda.synchronize()
+    ctx0 = reqs[0].fed
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sched.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(len(r.generated) >= warmup + steps for r in reqs)
+    while sched.step():
+        pass
+    return dt, ctx0 + (steps + 1) / 2.0
+
+
+def prefill_run(engine, tokens: int, repeats: int, seed: int):
+    """Seconds of one step that runs a whole `tokens`-token prompt (best of `repeats`)."""
+    import torch
+    from serve_amd.engine.batch import Segment
+    best = None
+    for i in range(repeats + 1):
+        prompt = random_prompts(1, tokens, engine.model.spec.vocab_size, seed + i)[0]
+        rid = f"prefill{i}"
+        assert engine.runner.admit(rid)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = engine.runner.step([Segment(rid, prompt, [tokens - 1])])
+        engine.sampler.sample(logits)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.runner.release(rid)
+        if i > 0:                                   # the first run loads and warms the libraries
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=16, help="fewer than 16 only to save time; both are reported")
+    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch-1/64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine
+
+    full_layers = 16
+    cfg = model_config(args.layers)
+    page = 16
+    pages_needed = args.batch * (-(-args.context // page)) + 64 * (-(-600 // page)) + 256
+    ecfg = EngineConfig(dtype="bfloat16", page_size=page, num_pages=pages_needed, max_context=args.context,
+                        max_requests=64, max_tokens_per_step=2048, prefill_chunk=2048, admission="reserve")
+    t_load = time.perf_counter()
+    engine = Engine.from_config(cfg, seed=0, cfg=ecfg)
+    print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
+
+    steps, warmup = args.steps, args.warmup
+    prompt_len = args.context - (warmup + steps + 3)
+    if prompt_len < 1:
+        print("bench.py: --steps + --warmup do not fit into the context")
+        return 2
+    dt, mean_ctx = decode_run(engine, args.batch, prompt_len, warmup, steps, seed=1)
+    ms_per_step = dt / steps * 1e3
+    value = args.batch * steps / dt
+    step_bytes = weight_bytes(cfg) + args.batch * mean_ctx * kv_bytes_per_token(cfg)
+    achieved = step_bytes / (dt / steps)
+    out = {
+        "metric": "decode tokens/s, Llama-3.2-1B shape, batch 8, context 4096, one MI355X",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+        "config": {"model": "llama-3.2-1b-shape", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single-gpu", "layers": args.layers, "layers_full": full_layers,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "page_size": page, "tied_embeddings": True, "rope_theta": cfg.rope_theta,
+                   "rope_scaling": "llama3 factor 32 low 1 high 4 orig 8192", "prefill_tokens": 2048},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    if not args.no_points:
+        T = 2048
+        pt = prefill_run(engine, T, repeats=3, seed=7)
+        out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                          "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}
+        points = {}
+        for b in (1, 64):
+            d, _ = decode_run(engine, b, 256, 4, 250, seed=10 + b)
+            points[f"decode_b{b}"] = round(b * 250 / d, 1)
+        out["points"] = points
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

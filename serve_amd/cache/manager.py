@@ -17,6 +17,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
+
 FREED = -1      # block-table entry of a page that the window has passed
 
 
@@ -84,6 +86,9 @@ class CacheManager:
         self.pools = [PagePool(n) for n in num_pages]
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
         self._requests: Dict[object, _Request] = {}
+        # the block tables once more as one int32 matrix per group, row = state slot, so that a
+        # step can gather the rows of its requests without walking Python lists
+        self.table_rows = [np.zeros((max_requests, max_pages_per_request), dtype=np.int32) for _ in windows]
 
     # -- queries --------------------------------------------------------------------------------
     @property
@@ -157,7 +162,10 @@ class CacheManager:
             return False
         for g, w in enumerate(wants):
             if w:
-                r.tables[g].extend(self.pools[g].take(w))
+                have = len(r.tables[g])
+                new = self.pools[g].take(w)
+                r.tables[g].extend(new)
+                self.table_rows[g][r.slot, have: have + w] = new
         r.tokens = max(r.tokens, n_tokens)
         return True
 
@@ -175,6 +183,7 @@ class CacheManager:
                 self.pools[g].give_back(gone)
                 for i in range(first):
                     table[i] = FREED
+                self.table_rows[g][r.slot, :first] = FREED
                 freed += len(gone)
         return freed
 
@@ -185,6 +194,7 @@ class CacheManager:
             raise CacheError(f"request {req_id!r} is released but not admitted")
         for g, table in enumerate(r.tables):
             self.pools[g].give_back([p for p in table if p != FREED])
+            self.table_rows[g][r.slot, : len(table)] = 0
         self._free_slots.append(r.slot)
 
     # -- self-check -------------------------------------------------------------------------------
@@ -201,6 +211,10 @@ class CacheManager:
                 raise CacheError(f"group {g}: a page is both free and held")
             if len(free) + len(held) != pool.num_pages:
                 raise CacheError(f"group {g}: {pool.num_pages - len(free) - len(held)} pages are lost")
+        for g in range(len(self.pools)):
+            for r in self._requests.values():
+                if self.table_rows[g][r.slot, : len(r.tables[g])].tolist() != r.tables[g]:
+                    raise CacheError(f"group {g}: the table matrix and the table of a request differ")
         slots = [r.slot for r in self._requests.values()]
         if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots):
             raise CacheError("a state slot is held twice")

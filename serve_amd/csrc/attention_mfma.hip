@@ -242,35 +242,36 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
 }
 
-// out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s
+// out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s; at most 64 splits.
+// One wave per (token, head): the lanes first share the work over the splits (weights), then over
+// the head dims (weighted sum, with independent loads that can all be in flight).
 __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o,
                                                           const float* __restrict__ part_ml,
                                                           bf16_t* __restrict__ out, int num_splits) {
+  __shared__ float wgt[64];
   const size_t item = blockIdx.x;                 // token * Hq + head
-  const float* ml = part_ml + item * num_splits * 2;
-  float M = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, ml[2 * s]);
-  float L = 0.f;
-  float o[(HD + 63) / 64];
-#pragma unroll
-  for (int a = 0; a < (HD + 63) / 64; ++a) o[a] = 0.f;
-  for (int s = 0; s < num_splits; ++s) {
-    const float ms = ml[2 * s];
-    if (ms == -INFINITY) continue;                // an empty split
-    const float w = __builtin_amdgcn_exp2f(ms - M);
-    L += ml[2 * s + 1] * w;
-    const float* po = part_o + (item * num_splits + s) * HD;
-#pragma unroll
-    for (int a = 0; a < (HD + 63) / 64; ++a) {
-      const int d = threadIdx.x + a * 64;
-      if (d < HD) o[a] += po[d] * w;
-    }
+  const int lane = threadIdx.x;
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < num_splits) {
+    ms = part_ml[(item * num_splits + lane) * 2];
+    ls = part_ml[(item * num_splits + lane) * 2 + 1];
   }
+  const float M = wave_max(ms);
+  const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - M);   // an empty split weighs 0
+  const float L = wave_sum(ls * w);
+  wgt[lane] = w;
+  __syncthreads();
   const float inv = 1.f / L;
+  const float* po = part_o + item * num_splits * HD;
 #pragma unroll
   for (int a = 0; a < (HD + 63) / 64; ++a) {
-    const int d = threadIdx.x + a * 64;
-    if (d < HD) out[item * HD + d] = from_float<bf16_t>(o[a] * inv);
+    const int d = lane + a * 64;
+    if (d < HD) {
+      float o = 0.f;
+#pragma unroll 8
+      for (int s = 0; s < num_splits; ++s) o += po[(size_t)s * HD + d] * wgt[s];
+      out[item * HD + d] = from_float<bf16_t>(o * inv);
+    }
   }
 }
 
@@ -292,7 +293,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
                                        int num_splits, float* part_o, float* part_ml, hipStream_t stream) {
   if (T <= 0 || B <= 0) return 0;
   if (D != HD || Hq <= 0 || Hk <= 0 || Hq % Hk || page_size <= 0 || (page_size & 3) || max_pages <= 0 ||
-      max_q_len <= 0 || num_splits < 1 || (q_stride & 7))
+      max_q_len <= 0 || num_splits < 1 || num_splits > 64 || (q_stride & 7))
     return SA_ERR_ARG;
   if (num_splits > 1 && (!part_o || !part_ml)) return SA_ERR_ARG;
   if ((long long)B * num_splits > 65535 || Hk > 65535) return SA_ERR_ARG;

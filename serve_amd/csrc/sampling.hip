@@ -22,21 +22,25 @@ __device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) 
   }
 }
 
-__global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ logits,
-                                                     const float* __restrict__ temperature,
-                                                     const unsigned long long* __restrict__ keys,
-                                                     int* __restrict__ out, int V) {
+// Stage 1: block (chunk, row) scans its chunk of the vocabulary and writes its best (score, index).
+__global__ __launch_bounds__(256) void sample_partial_kernel(const float* __restrict__ logits,
+                                                             const float* __restrict__ temperature,
+                                                             const unsigned long long* __restrict__ keys,
+                                                             float* __restrict__ part_v, int* __restrict__ part_i,
+                                                             int V, int chunk) {
   __shared__ float sv[4];
   __shared__ int si[4];
-  const int r = blockIdx.x;
+  const int r = blockIdx.y;
   const float* row = logits + (size_t)r * V;
   const float temp = temperature ? temperature[r] : 0.f;
   const bool greedy = !(temp > 0.f);
   const float inv_t = greedy ? 1.f : 1.f / temp;
   const unsigned long long key = greedy ? 0ull : keys[r];
+  const int lo = blockIdx.x * chunk;
+  const int hi = min(V, lo + chunk);
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
     float v = row[i];
     if (!greedy) {
       const unsigned int bits = (unsigned int)(mix64(key ^ (unsigned long long)i) >> 41);
@@ -60,15 +64,46 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < 4; ++w) take_better(bv, bi, sv[w], si[w]);
-    out[r] = bi == 0x7fffffff ? 0 : bi;
+    part_v[(size_t)r * gridDim.x + blockIdx.x] = bv;
+    part_i[(size_t)r * gridDim.x + blockIdx.x] = bi;
   }
 }
 
+// Stage 2: one wave per row picks the best of the chunks (ties still go to the lowest index).
+__global__ __launch_bounds__(64) void sample_final_kernel(const float* __restrict__ part_v,
+                                                          const int* __restrict__ part_i,
+                                                          int* __restrict__ out, int nchunks) {
+  const int r = blockIdx.x;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < nchunks; c += SA_WAVE)
+    take_better(bv, bi, part_v[(size_t)r * nchunks + c], part_i[(size_t)r * nchunks + c]);
+#pragma unroll
+  for (int o = SA_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, SA_WAVE);
+    const int oi = __shfl_xor(bi, o, SA_WAVE);
+    take_better(bv, bi, ov, oi);
+  }
+  if (threadIdx.x == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// how many chunks the vocabulary is cut into (the caller sizes the scratch arrays with it)
+extern "C" int sa_sample_chunks(int V) {
+  const int chunk = 2048;
+  int n = (V + chunk - 1) / chunk;
+  return n < 1 ? 1 : n;
+}
+
 extern "C" int sa_sample(const float* logits, const float* temperature, const unsigned long long* keys,
-                         int* out, int R, int V, hipStream_t stream) {
+                         int* out, float* part_v, int* part_i, int R, int V, hipStream_t stream) {
   if (R <= 0) return 0;
-  if (V <= 0) return SA_ERR_ARG;
-  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(256), 0, stream, logits, temperature, keys, out, V);
+  if (V <= 0 || R > 65535 || !part_v || !part_i) return SA_ERR_ARG;
+  const int nchunks = sa_sample_chunks(V);
+  const int chunk = (V + nchunks - 1) / nchunks;
+  hipLaunchKernelGGL(sample_partial_kernel, dim3(nchunks, R), dim3(256), 0, stream, logits, temperature, keys,
+                     part_v, part_i, V, chunk);
+  SA_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sample_final_kernel, dim3(R), dim3(64), 0, stream, part_v, part_i, out, nchunks);
   SA_LAUNCH_CHECK();
   return 0;
 }

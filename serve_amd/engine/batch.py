@@ -152,6 +152,28 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         MP = fixed_max_pages
     lay = StepLayout(T, B, R, MP, G)
     host = np.zeros(lay.total, dtype=np.int32)
+    if all(len(s.tokens) == 1 for s in segments):
+        # one token per request: fill the arrays without a Python loop over requests
+        n = B_real
+        slots_np = np.fromiter((cache.slot_of(s.req_id) for s in segments), dtype=np.int64, count=n)
+        before_np = np.asarray(before, dtype=np.int64)
+        host[lay.token_ids: lay.token_ids + n] = [s.tokens[0] for s in segments]
+        host[lay.positions: lay.positions + n] = before_np
+        host[lay.seg_of_token: lay.seg_of_token + B] = np.arange(B)
+        host[lay.cu_q: lay.cu_q + B + 1] = np.arange(B + 1)
+        host[lay.ctx_len: lay.ctx_len + B] = 1
+        host[lay.ctx_len: lay.ctx_len + n] = before_np + 1
+        host[lay.state_slots: lay.state_slots + n] = slots_np
+        host[lay.logit_rows: lay.logit_rows + R] = [i for i, s in enumerate(segments) if len(s.want)]
+        for g in range(G):
+            rows = cache.table_rows[g][slots_np]
+            host[lay.block_tables[g]: lay.block_tables[g] + n * MP].reshape(n, MP)[:] = rows[:, :MP]
+            host[lay.slots[g]: lay.slots[g] + B] = -1
+            host[lay.slots[g]: lay.slots[g] + n] = rows[np.arange(n), before_np // ps] * ps + before_np % ps
+        ctx_lens = [b + 1 for b in before] + [1] * pad
+        facts = dict(q_lens=[1] * B, ctx_lens=ctx_lens, max_q_len=1, max_ctx_len=max(ctx_lens),
+                     max_pages=MP, decode_only=True)
+        return lay, host, facts
     cu = 0
     r_i = 0
     q_lens, ctx_lens = [], []

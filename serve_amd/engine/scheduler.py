@@ -247,7 +247,7 @@ class Scheduler:
         for r, n, s in zip(plan.requests, plan.counts, plan.samples):
             toks = r.all_tokens()[r.fed: r.fed + n]
             segments.append(Segment(r.req_id, toks, [n - 1] if s else []))
-        logits = self.runner.step(segments)
+        logits = self.runner.step(segments, borrow=True)     # sampled from before the next step
         samplers = [r for r, s in zip(plan.requests, plan.samples) if s]
         tokens = self.sampler.sample(logits, [r.temperature for r in samplers],
                                      [r.req_id for r in samplers], [len(r.generated) for r in samplers])

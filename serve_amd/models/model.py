@@ -96,6 +96,10 @@ class Model:
         """Per cache layer: the fixed-size per-request state its mixer needs."""
         return [self.layers[l].mixer.state_request() for l in self._cache_writer_layer]
 
+    def graph_safe(self) -> bool:
+        """Whether every part only enqueues GPU work, so that a step can be captured into a graph."""
+        return all(getattr(p, "graph_safe", False) for p in self._owners().values())
+
     # -- loading ------------------------------------------------------------------------------
     def load(self, tensors_by_owner: Dict[str, Dict[str, torch.Tensor]], rt: Runtime) -> None:
         self.rt = rt

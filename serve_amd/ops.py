@@ -208,8 +208,12 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Opti
         _check(temperature.dtype == torch.float32 and temperature.numel() == R, "temperature must be fp32 [R]")
         _check(keys is not None and keys.dtype == torch.int64 and keys.numel() == R, "keys must be int64 [R]")
     lib = load_library("sampling")
-    _ret(lib.sa_sample(_ptr(logits), _ptr(temperature), _ptr(keys), _ptr(out), c_int(R), c_int(V), _stream()),
-         "sample")
+    _check(R <= 65535, "at most 65535 rows are sampled in one call")
+    nchunks = lib.sa_sample_chunks(c_int(V))
+    part_v = torch.empty((R, nchunks), dtype=torch.float32, device=logits.device)
+    part_i = torch.empty((R, nchunks), dtype=torch.int32, device=logits.device)
+    _ret(lib.sa_sample(_ptr(logits), _ptr(temperature), _ptr(keys), _ptr(out), _ptr(part_v), _ptr(part_i),
+                       c_int(R), c_int(V), _stream()), "sample")
     return out
 
 
@@ -282,8 +286,16 @@ def attention_splits(decode_only: bool, num_segments: int, num_kv_heads: int, ma
     about 2048 waves in all, and no part shorter than 128 keys."""
     if not decode_only:
         return 1
-    by_length = max(1, max_ctx_len // 128)
-    by_waves = max(1, 2048 // max(1, num_segments * num_kv_heads))
+    # both inputs are rounded up to powers of two, so that a step run eagerly and the same step
+    # replayed from a graph (padded batch, context bucket) cut the keys alike
+    ctx = 256
+    while ctx < max_ctx_len:
+        ctx *= 2
+    segs = 1
+    while segs < num_segments:
+        segs *= 2
+    by_length = max(1, ctx // 128)
+    by_waves = max(1, 2048 // (segs * num_kv_heads))
     return max(1, min(by_length, by_waves, 64))
 
 

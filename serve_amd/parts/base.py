@@ -86,6 +86,10 @@ class Runtime:
 class Part:
     """Base of all parts."""
 
+    # whether `forward` only enqueues GPU work on the current stream (no read-back to the host,
+    # no host-side branching on device data): only then can a step be captured into a HIP graph
+    graph_safe = False
+
     def param_requests(self) -> List[ParamRequest]:
         return []
 

@@ -23,6 +23,8 @@ class RMSNorm(Part):
     """y = x * rsqrt(mean(x^2) + eps) * weight (serve/model.py:57-68), fused with the addition
     of the previous part's output into the fp32 residual stream (serve/model.py:147-148)."""
 
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size, self.eps = int(size), float(eps)
 
@@ -74,6 +76,8 @@ class RotaryPosition(Part):
     (serve/hf_utils/convert_hf_checkpoint.py:115-118), which is `pairing="adjacent"`.
     `rot_dim < head_dim` leaves the remaining dims of every head as they are."""
 
+    graph_safe = True
+
     def __init__(self, head_dim: int, rot_dim: int, theta: float, scaling: Optional[dict] = None,
                  pairing: str = "half"):
         if pairing not in ("half", "adjacent"):
@@ -102,6 +106,8 @@ class RotaryPosition(Part):
 class GQAAttention(Part):
     """q, k, v in one product, rotate q and k, store k and v in the paged cache, attend over the
     cache, project back (serve/model.py:88-134).  Query head h reads KV head h // (Hq // Hk)."""
+
+    graph_safe = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
                  position: PartSpec, window: Optional[int] = None):
@@ -156,6 +162,8 @@ class SwiGLU(Part):
     """down(silu(gate x) * up x), no biases (serve/model.py:71-85); gate and up run as one
     product over the stacked matrix."""
 
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
 
@@ -188,6 +196,8 @@ class SwiGLU(Part):
 class TokenEmbedding(Part):
     """x = table[token] (serve/model.py:157,220); the residual stream it starts is fp32."""
 
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
 
@@ -206,6 +216,8 @@ class TokenEmbedding(Part):
 class LinearHead(Part):
     """logits = h @ W^T in fp32 (serve/model.py:159,226-231).  A tied head has no tensor of its
     own: the model hands it the embedding table (serve/hf_utils/convert_hf_checkpoint.py:146-147)."""
+
+    graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)

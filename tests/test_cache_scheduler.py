@@ -172,7 +172,7 @@ class FakeRunner:
         self.cache.release(rid)
         del self.history[rid]
 
-    def step(self, segments):
+    def step(self, segments, borrow=False):
         lay, host, facts = plan_step(segments, self.cache, VOCAB)      # allocates as the real step does
         out = []
         for i, s in enumerate(segments):

@@ -1,0 +1,363 @@
+"""Generation through the entry point, the parts alone, trace replay as a program, and a toy
+mixer with state of its own that is registered, built and stepped from the test."""
+from __future__ import annotations
+
+import json
+import os
+import random
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import util
+from tests.plain import llama_plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ---------------------------------------------------------------------------------------------
+# the entry point in the reference's manner: load_model / Request / generate
+# ---------------------------------------------------------------------------------------------
+def test_greedy_generation_tiny_a_whole_prompts(tmp_path):
+    """Tiny A's workload: prompts of 7, 13 and 1 tokens, 8 greedy steps each, page size 4."""
+    import serve_amd
+    folder = util.make_folder(tmp_path, "A")
+    model = serve_amd.load_model(folder, "cuda", torch.float32, page_size=4, num_pages=64, max_context=64,
+                                 max_requests=4)
+    rng = random.Random(0)
+    prompts = [util.random_tokens(rng, n, 256) for n in (7, 13, 1)]
+    reqs = [serve_amd.Request(torch.tensor(p), len(p), 8) for p in prompts]
+    out = serve_amd.generate(model, reqs, temperature=0.0, return_logits=True)
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    for p, r in zip(prompts, out):
+        want = llama_plain.generate(p, 8, w, cfg)
+        assert r.generated_tokens.tolist() == want
+        assert r.generated_tokens.dtype == torch.long and r.input_length == len(p)
+        # the logits kept are those of the last step (serve/run.py:229-230)
+        last = llama_plain.forward(p + want[:-1], w, cfg)[-1]
+        util.assert_close(r.logits.reshape(-1), last, "float32", "last-step logits")
+    assert not model.runner.cache.live_requests()
+    model.runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sampled_generation_tiny_b_chunked_beside_decodes(tmp_path, dtype):
+    """Tiny B's workload: prompts of 5, 17, 30 and 2 tokens prefilled in chunks of 8 beside decoding
+    requests, 6 draws at temperature 0.8 with a fixed sampler seed, page size 8.  Each draw must be
+    the plain sampler's draw from the engine's own logits path: teacher-forced on the engine's
+    tokens, the plain logits give the same token unless two scores are within the dtype's error."""
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine, Request
+    folder = util.make_folder(tmp_path, "B")
+    eng = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=8, num_pages=24, max_context=64,
+                                                 max_requests=4, prefill_chunk=8, max_tokens_per_step=12, seed=77))
+    rng = random.Random(1)
+    prompts = [util.random_tokens(rng, n, 509) for n in (5, 17, 30, 2)]
+    out = eng.generate([Request(torch.tensor(p), len(p), 6) for p in prompts], temperature=0.8)
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    margin = 1e-4 if dtype == "float32" else 5e-2
+    for rid, (p, r) in enumerate(zip(prompts, out)):
+        got = r.generated_tokens.tolist()
+        assert len(got) == 6
+        seq = list(p)
+        for i, t in enumerate(got):
+            logits = llama_plain.forward(seq, w, cfg)[-1]
+            noise = llama_plain.exponential_noise(77, rid, i, 509).double()
+            score = logits / 0.8 - noise.log()
+            assert score.max() - score[t] <= margin, f"request {rid} token {i}: {t} is not the draw"
+            seq.append(t)
+    # the same requests one at a time give the same tokens: draws do not depend on the batch
+    eng2 = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=8, num_pages=24, max_context=64,
+                                                  max_requests=4, seed=77))
+    alone = eng2.generate([Request(torch.tensor(prompts[0]), len(prompts[0]), 6)], temperature=0.8)
+    if dtype == "float32":
+        assert alone[0].generated_tokens.tolist() == out[0].generated_tokens.tolist()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_few_pages_preemption_gives_the_same_tokens(tmp_path, dtype):
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine, Request
+    folder = util.make_folder(tmp_path, "C")
+    rng = random.Random(2)
+    prompts = [util.random_tokens(rng, n, 1000) for n in (20, 9, 33, 14)]
+
+    def run(admission, num_pages):
+        eng = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=8, num_pages=num_pages, max_context=96,
+                                                     max_requests=4, admission=admission))
+        out = eng.generate([Request(torch.tensor(p), len(p), 24) for p in prompts])
+        eng.runner.cache.check_invariants()
+        assert eng.runner.cache.free_pages() == num_pages
+        return [r.generated_tokens.tolist() for r in out]
+    roomy = run("reserve", 64)
+    assert run("reserve", 12) == roomy              # 96 tokens of cache: requests wait their turn
+    assert run("optimistic", 12) == roomy           # pages run out while decoding: preempt and recompute
+
+
+def test_graph_replays_equal_eager_steps(tmp_path):
+    """Decode steps replayed from a captured graph, with eager work between replays, equal the
+    same steps run eagerly, replay after replay."""
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    folder = util.make_folder(tmp_path, "C")
+    rng = random.Random(3)
+    toks = {k: util.random_tokens(rng, 90, 1000) for k in "abc"}
+    results = {}
+    for use_graphs in (False, True):
+        eng = Engine.from_folder(folder, EngineConfig(dtype="bfloat16", page_size=16, num_pages=32, max_context=128,
+                                                     max_requests=4, use_graphs=use_graphs))
+        rows = []
+        for k in toks:
+            eng.runner.admit(k)
+        eng.step([Segment(k, toks[k][:40], []) for k in toks])
+        for i in range(40, 90):
+            if i % 7 == 0:                  # eager work of another shape between the replays
+                eng.runner.admit("x")
+                eng.step([Segment("x", toks["a"][:5], [4])])
+                eng.runner.release("x")
+                torch.cuda.synchronize()
+            rows.append(eng.step([Segment(k, [toks[k][i]], [0]) for k in toks]).cpu())
+        results[use_graphs] = torch.stack(rows)
+    assert torch.equal(results[False], results[True])
+
+
+# ---------------------------------------------------------------------------------------------
+# each part alone
+# ---------------------------------------------------------------------------------------------
+def runtime(dtype):
+    from serve_amd.parts.base import Runtime
+    return Runtime(torch.device(DEV), dtype)
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_part_rmsnorm(dtype):
+    from serve_amd.parts.standard import RMSNorm
+    part = RMSNorm(size=88, eps=1e-6)
+    w = rnd((88,), dtype, 1) * 0.1 + 1
+    part.load({"weight": w}, runtime(dtype))
+    x = rnd((5, 88), torch.float32, 2)
+    delta = rnd((5, 88), dtype, 3)
+    x0 = x.clone()
+    y = part.forward(x, delta)
+    want = llama_plain.rms_norm(x0.double() + delta.double(), w.double(), 1e-6)
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(y.double(), want, **tol)
+    torch.testing.assert_close(x.double(), x0.double() + delta.double(), atol=1e-6, rtol=1e-6)
+
+
+def test_part_rope_frequencies_equal_the_plain_ones():
+    from serve_amd.parts.standard import rope_inverse_frequencies
+    for cfg in (util.TINY_A, util.TINY_B, util.TINY_C):
+        sc = None if cfg.rope_scaling is None else cfg.rope_scaling.to_hf_dict()
+        got = rope_inverse_frequencies(cfg.head_dim, cfg.rope_theta, sc)
+        want = llama_plain.rope_frequencies(cfg.head_dim, cfg.rope_theta, sc)
+        assert got.dtype == torch.float32
+        torch.testing.assert_close(got, want, atol=0, rtol=2e-7)
+    big = dict(factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)
+    torch.testing.assert_close(rope_inverse_frequencies(64, 500000.0, big),
+                               llama_plain.rope_frequencies(64, 500000.0, big), atol=0, rtol=2e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_part_swiglu(dtype):
+    from serve_amd.parts.standard import SwiGLU
+    part = SwiGLU(hidden_size=72, intermediate_size=200)
+    t = {"gate_proj.weight": rnd((200, 72), dtype, 1, 0.1), "up_proj.weight": rnd((200, 72), dtype, 2, 0.1),
+         "down_proj.weight": rnd((72, 200), dtype, 3, 0.1)}
+    part.load(dict(t), runtime(dtype))
+    for rows in (3, 70):                              # few rows: fused kernel; many: product then gate
+        h = rnd((rows, 72), dtype, 4)
+        got = part.forward(h, None)
+        want = llama_plain.swiglu(h.double(), *(t[k].double() for k in
+                                                ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
+        tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=3e-2, rtol=2e-2)
+        torch.testing.assert_close(got.double(), want, **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_part_attention_whole_and_in_portions(dtype):
+    """The mixer alone, driven through a cache and step contexts built by hand: the plain
+    attention part on the whole sequence equals the mixer fed in two portions."""
+    from serve_amd.cache.manager import CacheManager
+    from serve_amd.cache.storage import CacheStorage
+    from serve_amd.config.spec import PartSpec
+    from serve_amd.engine.batch import Segment, build_step
+    from serve_amd.parts.standard import GQAAttention
+    d, Hq, Hk, D, S = 80, 6, 2, 32, 29
+    rt = runtime(dtype)
+    pos = PartSpec("rope", dict(head_dim=D, rot_dim=D, theta=10000.0, scaling=None, pairing="half"))
+    part = GQAAttention(hidden_size=d, num_heads=Hq, num_kv_heads=Hk, head_dim=D, scale=D ** -0.5, position=pos)
+    names = {"q_proj.weight": (Hq * D, d), "k_proj.weight": (Hk * D, d), "v_proj.weight": (Hk * D, d),
+             "o_proj.weight": (d, Hq * D)}
+    t = {k: rnd(s, dtype, i, 0.1) for i, (k, s) in enumerate(names.items())}
+    part.load(dict(t), rt)
+    cache = CacheManager([None], [8], 8, 2, 8)
+    storage = CacheStorage(rt, [part.cache_request()], [None], [None], [8], 8, 2)
+    cache.admit("r")
+    h = rnd((S, d), dtype, 9)
+    outs = []
+    for lo, hi in ((0, 11), (11, S)):
+        ctx = build_step([Segment("r", [0] * (hi - lo), [])], cache, 10, rt.device)
+        outs.append(part.forward(h[lo:hi].contiguous(), ctx, storage.layers[0], True))
+    got = torch.cat(outs)
+    w = {"p.self_attn." + k: v.cpu() for k, v in t.items()}
+    cfg = dict(num_attention_heads=Hq, num_key_value_heads=Hk, head_dim=D, hidden_size=d, rope_theta=10000.0)
+    want = llama_plain.attention_part(h.double().cpu(), w, "p.", cfg, torch.arange(S))
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=3e-2, rtol=2e-2)
+    torch.testing.assert_close(got.double().cpu(), want, **tol)
+
+
+# ---------------------------------------------------------------------------------------------
+# trace replay as a program
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    folder = util.make_folder(tmp_path, "B")
+    rng = random.Random(5)
+    a, b = util.random_tokens(rng, 40, 509), util.random_tokens(rng, 21, 509)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": [0, 16]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[17:19], "want": []}, {"id": "b", "tokens": b[:20], "want": [19]}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[20:], "want": [0]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[19:], "want": list(range(21))}], "end": ["a"]},
+    ]
+    out = tmp_path / f"out_{dtype}"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", "128"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+                          timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    pa, pb = util.plain_logits(folder, a), util.plain_logits(folder, b)
+
+    def read(step, rows):
+        arr = np.fromfile(out / f"{step}.f32", dtype="<f4")
+        return torch.from_numpy(arr.reshape(rows, 509))
+    util.assert_close(read(0, 2), pa[[0, 16]], dtype, "step 0")
+    util.assert_close(read(1, 1), pb[[19]], dtype, "step 1")
+    util.assert_close(read(2, 1), pb[[20]], dtype, "step 2")
+    util.assert_close(read(3, 21), pa[19:], dtype, "step 3")
+
+
+# ---------------------------------------------------------------------------------------------
+# a toy mixer with state of its own, defined here, registered, built and stepped
+# ---------------------------------------------------------------------------------------------
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    """A mixer that keeps, per request, the running sum of the activations it has seen
+    (out[t] = proj(sum of h[0..t])): state of fixed size, no paged cache.  It lives in this test
+    only; the framework's files are not touched.  Fed whole or in portions, beside another
+    request, its logits must be the same, which needs the state slots to be zeroed at admission,
+    kept between steps and separated between requests."""
+    from dataclasses import dataclass
+
+    import serve_amd
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.spec import LayerSpec, ModelSpec, PartSpec, RunEntry
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    from serve_amd.parts.base import ParamRequest, Part, StateRequest
+    from serve_amd.parts.linear import linear
+    from serve_amd.weights.loader import write_random_model
+
+    class RunningSumMixer(Part):
+        def __init__(self, hidden_size):
+            self.hidden_size = hidden_size
+
+        def param_requests(self):
+            return [ParamRequest("proj.weight", (self.hidden_size, self.hidden_size))]
+
+        def state_request(self):
+            return StateRequest((self.hidden_size,), torch.float32)
+
+        def load(self, tensors, rt):
+            self.rt, self.w = rt, tensors["proj.weight"]
+
+        def forward(self, h, ctx, cache, writes_cache=True):
+            out = torch.empty_like(h, dtype=torch.float32)
+            cu = [0]
+            for n in ctx.q_lens:
+                cu.append(cu[-1] + n)
+            slots = ctx.state_slots.tolist()
+            for i, slot in enumerate(slots[: len(ctx.q_lens)]):
+                seg = h[cu[i]: cu[i + 1]].float()
+                run = torch.cumsum(seg, dim=0) + cache.state[slot]
+                cache.state[slot] = run[-1]
+                out[cu[i]: cu[i + 1]] = run
+            return linear(out.to(h.dtype).contiguous(), self.w)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int = 50
+        hidden_size: int = 32
+        num_hidden_layers: int = 2
+        architecture = "ToyRunningSumLM"
+
+        def to_hf_dict(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size,
+                    "hidden_size": self.hidden_size, "num_hidden_layers": self.num_hidden_layers}
+
+        @staticmethod
+        def from_hf_dict(d):
+            return ToyConfig(d["vocab_size"], d["hidden_size"], d["num_hidden_layers"])
+
+    def build(cfg):
+        norm = PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": 1e-5})
+        layers = []
+        for i in range(cfg.num_hidden_layers):
+            p = f"toy.{i}."
+            layers.append(LayerSpec(
+                mixer=PartSpec("running_sum", {"hidden_size": cfg.hidden_size}),
+                ffn=PartSpec("swiglu", {"hidden_size": cfg.hidden_size, "intermediate_size": 48}),
+                mixer_norm=norm, ffn_norm=norm,
+                weights={"mixer.proj.weight": p + "proj", "ffn.gate_proj.weight": p + "gate",
+                         "ffn.up_proj.weight": p + "up", "ffn.down_proj.weight": p + "down",
+                         "mixer_norm.weight": p + "n1", "ffn_norm.weight": p + "n2"}))
+        return ModelSpec(architecture=cfg.architecture, vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
+                         embedding=PartSpec("token_embedding", {"vocab_size": cfg.vocab_size,
+                                                                "hidden_size": cfg.hidden_size}),
+                         layers=layers, run_order=[RunEntry(i, i) for i in range(cfg.num_hidden_layers)],
+                         final_norm=norm,
+                         lm_head=PartSpec("linear_head", {"vocab_size": cfg.vocab_size,
+                                                          "hidden_size": cfg.hidden_size, "tied": True}),
+                         weights={"embedding.weight": "toy.embed", "final_norm.weight": "toy.norm",
+                                  "lm_head.weight": "toy.head"})
+
+    serve_amd.register_part("mixer", "running_sum", RunningSumMixer)
+    serve_amd.register_architecture("ToyRunningSumLM", ToyConfig.from_hf_dict, build)
+    folder = write_random_model(str(tmp_path / "toy"), ToyConfig(), seed=3)
+    eng = Engine.from_folder(folder, EngineConfig(dtype="float32", page_size=8, num_pages=8, max_context=64,
+                                                 max_requests=3))
+    assert eng.runner.windows == [] and eng.runner.storage.layers[0].state.shape == (3, 32)
+    rng = random.Random(4)
+    a, b = util.random_tokens(rng, 12, 50), util.random_tokens(rng, 7, 50)
+
+    def whole(tokens):
+        eng.runner.admit("w")
+        out = eng.step([Segment("w", tokens, list(range(len(tokens))))])
+        eng.runner.release("w")
+        return out
+    wa, wb = whole(a), whole(b)
+    eng.runner.admit("a")
+    eng.runner.admit("b")
+    r1 = eng.step([Segment("a", a[:5], list(range(5))), Segment("b", b[:1], [0])])
+    r2 = eng.step([Segment("b", b[1:], list(range(6))), Segment("a", a[5:7], [0, 1])])
+    r3 = eng.step([Segment("a", a[7:], list(range(5)))])
+    got_a = torch.cat([r1[:5], r2[6:], r3])
+    got_b = torch.cat([r1[5:], r2[:6]])
+    torch.testing.assert_close(got_a, wa, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(got_b, wb, atol=1e-5, rtol=1e-5)
+    assert not torch.allclose(wa[-1], wb[-1])
+    # the state matters: the last position differs from running the last token alone
+    assert not torch.allclose(whole(a[-1:])[0], wa[-1], atol=1e-3)

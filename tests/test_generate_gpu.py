@@ -94,8 +94,21 @@ def test_few_pages_preemption_gives_the_same_tokens(tmp_path, dtype):
         assert eng.runner.cache.free_pages() == num_pages
         return [r.generated_tokens.tolist() for r in out]
     roomy = run("reserve", 64)
-    assert run("reserve", 12) == roomy              # 96 tokens of cache: requests wait their turn
-    assert run("optimistic", 12) == roomy           # pages run out while decoding: preempt and recompute
+    waiting = run("reserve", 12)                    # 96 tokens of cache: requests wait their turn
+    preempting = run("optimistic", 12)              # pages run out while decoding: preempt and recompute
+    if dtype == "float32":
+        assert waiting == roomy and preempting == roomy
+    else:
+        # in bfloat16 another batch composition rounds differently, and a random model has many
+        # nearly equal logits: every run's tokens must be best tokens of the plain model
+        w, cfg = util.plain_weights(folder), util.plain_config(folder)
+        for run_tokens in (roomy, waiting, preempting):
+            for p, got in zip(prompts, run_tokens):
+                seq = list(p)
+                for t in got:
+                    logits = llama_plain.forward(seq, w, cfg)[-1]
+                    assert logits.max() - logits[t] <= 2e-2
+                    seq.append(t)
 
 
 def test_graph_replays_equal_eager_steps(tmp_path):

@@ -1,0 +1,103 @@
+"""Command line: `python -m serve_amd <command>`.
+
+    generate      token ids in, generated token ids out (JSON lines)
+    random-model  write a model folder with random weights for a named shape or a config.json
+    replay        the trace replay program (same as bin/trace_run)
+    benchmark     the offline batch benchmark (same as python -m serve_amd.benchmark)
+
+Option names follow the reference where it has them: `temperature`, `max_new_tokens`
+(serve/run.py:20,242), dtype (serve/utils.py:41); the rest name the engine settings the
+reference keeps as literals in its code.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+
+def _generate(argv) -> int:
+    ap = argparse.ArgumentParser(prog="python -m serve_amd generate")
+    ap.add_argument("--model", required=True, help="model folder (config.json + model.safetensors)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--prompt-ids", help="file with one prompt a line: JSON list or blank-separated token ids "
+                    "(default: standard input)")
+    ap.add_argument("--max-new-tokens", type=int, default=32)
+    ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy (serve/run.py:56-57)")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--num-pages", type=int, default=None)
+    ap.add_argument("--memory-fraction", type=float, default=0.6)
+    ap.add_argument("--max-context", type=int, default=4096)
+    ap.add_argument("--max-requests", type=int, default=256)
+    ap.add_argument("--max-tokens-per-step", type=int, default=2048)
+    ap.add_argument("--prefill-chunk", type=int, default=2048)
+    ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")
+    args = ap.parse_args(argv)
+    import torch
+
+    from .config.engine import EngineConfig
+    from .engine.engine import Engine, Request
+    src = open(args.prompt_ids) if args.prompt_ids else sys.stdin
+    prompts = []
+    for line in src:
+        line = line.strip()
+        if line:
+            prompts.append(json.loads(line) if line.startswith("[") else [int(t) for t in line.split()])
+    cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, num_pages=args.num_pages,
+                       memory_fraction=args.memory_fraction, max_context=args.max_context,
+                       max_requests=args.max_requests, max_tokens_per_step=args.max_tokens_per_step,
+                       prefill_chunk=args.prefill_chunk, admission=args.admission, seed=args.seed)
+    engine = Engine.from_folder(args.model, cfg)
+    out = engine.generate([Request(torch.tensor(p, dtype=torch.long), len(p), args.max_new_tokens) for p in prompts],
+                          temperature=args.temperature)
+    for r in out:
+        print(json.dumps(r.generated_tokens.tolist()), flush=True)
+    return 0
+
+
+def _random_model(argv) -> int:
+    ap = argparse.ArgumentParser(prog="python -m serve_amd random-model")
+    ap.add_argument("--out", required=True, help="folder to write config.json and model.safetensors into")
+    g = ap.add_mutually_exclusive_group(required=True)
+    g.add_argument("--shape", help="a named shape (tiny, llama-1b, llama-3b, llama-8b)")
+    g.add_argument("--config", help="a config.json to take the sizes from")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args(argv)
+    from .weights.loader import write_random_model
+    if args.shape:
+        from .benchmark import SHAPES
+        if args.shape not in SHAPES:
+            ap.error(f"unknown shape {args.shape!r}; known: {sorted(SHAPES)}")
+        config = SHAPES[args.shape]
+    else:
+        from .registry import get_architecture
+        with open(args.config) as f:
+            raw = json.load(f)
+        config = get_architecture(raw["architectures"][0]).config_from_dict(raw)
+    write_random_model(args.out, config, args.seed)
+    print(args.out)
+    return 0
+
+
+def main(argv=None) -> int:
+    argv = list(sys.argv[1:] if argv is None else argv)
+    commands = {"generate": _generate, "random-model": _random_model}
+    if not argv or argv[0] in ("-h", "--help"):
+        print(__doc__)
+        return 0
+    cmd, rest = argv[0], argv[1:]
+    if cmd == "replay":
+        from .engine.replay import main as replay_main
+        return replay_main(rest)
+    if cmd == "benchmark":
+        from .benchmark import main as bench_main
+        return bench_main(rest)
+    if cmd not in commands:
+        print(f"unknown command {cmd!r}; known: generate, random-model, replay, benchmark", file=sys.stderr)
+        return 2
+    return commands[cmd](rest)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

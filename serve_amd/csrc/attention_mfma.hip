@@ -17,10 +17,12 @@
 // MFMA use (v_mfma_f32_16x16x32_bf16: D[i][j] += sum_k A[i][k] B[k][j]; lane l holds A row l%16,
 // B column l%16, k-slots 8*(l/16)..+7, and D[4*(l/16)+r][l%16]):
 //   S^T = K Q^T : A = 16 keys x 32 dims of K (16-byte loads along D), B = Q^T.  A lane then holds,
-//                 for ITS query column, keys 4g..4g+3 of both 16-key halves: exactly the eight
-//                 k-slots it must supply for the next product, so P never moves between lanes.
+//                 for ITS query column, the scores of eight keys: exactly the eight k-slots it
+//                 must supply for the next product, so P never moves between lanes.  The keys of
+//                 a block are dealt to the tile rows so that those eight keys are consecutive.
 //   O^T = V^T P^T: A = 16 dims x 32 keys of V^T.  Values are stored transposed inside a page
-//                 ([Hk, D, page_size]), so four consecutive keys at one dim are one 8-byte load.
+//                 ([Hk, D, page_size]), so eight consecutive keys at one dim are one 16-byte load
+//                 (two 8-byte loads when the page size is a multiple of 4 only).
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -42,17 +44,25 @@ constexpr int DC = (HD + 31) / 32;   // 32-wide chunks of the head dim for Q K^T
 constexpr int DT = HD / 16;          // 16-wide tiles of the head dim for P V
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 128, "head size must be a multiple of 16 up to 128");
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// two floats to two bf16 (round to nearest even) in one v_cvt_pk_bf16_f32
 __device__ __forceinline__ uint32_t pack2bf(float a, float b) {
-  return (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+  const float2_t f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
-template <int NT>
+// NT: column tiles (16 query rows each) per wave.  POW2: the page size is a power of two of at
+// least 8 (key -> page by shift, 16-byte value runs); otherwise any multiple of 4 (division,
+// 8-byte value runs).
+template <int NT, bool POW2>
 __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
-    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, float scale_log2e, int window,
-    int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
+    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
   const int c = lane & 15;
@@ -113,7 +123,64 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
 
   const size_t k_page_stride = (size_t)Hk * page_size * HD;   // elements per page (K and V alike)
-  for (int kb = b0; kb < b1; ++kb) {
+  constexpr bool wide_v = POW2;                                // 8 consecutive keys lie in one page
+
+  // Which key sits in which row of the two 16-key tiles is free to choose.  Row i of tile t holds
+  // key 8*(i/4) + 4*t + (i%4) of the block, so that after S^T = K Q^T lane group g holds the
+  // scores of keys 8g .. 8g+7: one 16-byte run of V^T per dim when a page holds a multiple of 8 keys.
+  struct Block {
+    Frag kf[2][DC];
+    Frag vf[DT];
+  };
+  // key index -> (page, offset in the page); a shift when the page size is a power of two
+  auto locate = [&](int key, int& page, int& off) {
+    int idx;
+    if (POW2) {
+      idx = key >> page_shift;
+      off = key & (page_size - 1);
+    } else {
+      idx = key / page_size;
+      off = key - idx * page_size;
+    }
+    page = max(bt[idx], 0);
+  };
+  auto load_block = [&](int kb, Block& blk) {
+    const int key0 = kb << 5;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int kk = min(key0 + 8 * (c >> 2) + 4 * t + (c & 3), ctx - 1);
+      int page, off;
+      locate(kk, page, off);
+      const bf16_t* kp = k_pages + (size_t)page * k_page_stride + ((size_t)hk * page_size + off) * HD;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        blk.kf[t][dc].u = make_uint4(0, 0, 0, 0);
+        if (dc * 32 + g * 8 < HD) blk.kf[t][dc].u = *reinterpret_cast<const uint4*>(kp + dc * 32 + g * 8);
+      }
+    }
+    if (wide_v) {
+      const int run = min(key0 + 8 * g, (ctx - 1) & ~7);
+      int page, off;
+      locate(run, page, off);
+      const bf16_t* vp = v_pages + (size_t)page * k_page_stride + (size_t)hk * HD * page_size + off;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        blk.vf[dt].u = *reinterpret_cast<const uint4*>(vp + (size_t)(dt * 16 + c) * page_size);
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int run = min(key0 + 8 * g + 4 * h, (ctx - 1) & ~3);
+        int page, off;
+        locate(run, page, off);
+        const bf16_t* vp = v_pages + (size_t)page * k_page_stride + (size_t)hk * HD * page_size + off;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          blk.vf[dt].h[h] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * page_size);
+      }
+    }
+  };
+
+  auto compute = [&](int kb, Block& blk) {
     const int key0 = kb << 5;
     // every key of the block visible to every row of the tile: no masking needed
     const bool full = (key0 + 31 <= ctx_before + j_lo) && (window <= 0 || key0 > ctx_before + j_hi - window);
@@ -121,44 +188,29 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     // ---- S^T = K Q^T --------------------------------------------------------------------
     floatx4_t s[2][NT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int kk = min(key0 + t * 16 + c, ctx - 1);
-      const int page = max(bt[kk / page_size], 0);
-      const bf16_t* kp = k_pages + (size_t)page * k_page_stride + ((size_t)hk * page_size + kk % page_size) * HD;
-      Frag kf[DC];
-#pragma unroll
-      for (int dc = 0; dc < DC; ++dc) {
-        kf[dc].u = make_uint4(0, 0, 0, 0);
-        if (dc * 32 + g * 8 < HD) kf[dc].u = *reinterpret_cast<const uint4*>(kp + dc * 32 + g * 8);
-      }
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int n = 0; n < NT; ++n) {
         s[t][n] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc)
-          s[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[dc].v, qf[n][dc].v, s[t][n], 0, 0, 0);
+          s[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[t][dc].v, qf[n][dc].v, s[t][n], 0, 0, 0);
       }
-    }
 
-    // ---- V^T fragments (issued early so that the loads overlap the softmax) --------------
-    Frag vf[DT];
+    if (!full) {
+      // keys at or beyond the end of the context hold whatever the page held before: their
+      // probability is 0, and 0 times such a value must stay 0
+      const int first = key0 + 8 * g;
+      uint32_t keep[4];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int run = key0 + h * 16 + 4 * g;                 // first of this lane's 4 keys
-      const int runc = min(run, (ctx - 1) & ~3);
-      const int page = max(bt[runc / page_size], 0);
-      const bf16_t* vp = v_pages + (size_t)page * k_page_stride + (size_t)hk * HD * page_size + runc % page_size;
+      for (int i = 0; i < 4; ++i)
+        keep[i] = (first + 2 * i < ctx ? 0x0000ffffu : 0u) | (first + 2 * i + 1 < ctx ? 0xffff0000u : 0u);
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-        vf[dt].h[h] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * page_size);
-      if (!full) {
-        // keys at or beyond the end of the context hold whatever the page held before
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (run + i >= ctx) {
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vf[dt].s[h * 4 + i] = 0;
-          }
+      for (int dt = 0; dt < DT; ++dt) {
+        blk.vf[dt].u.x &= keep[0];
+        blk.vf[dt].u.y &= keep[1];
+        blk.vf[dt].u.z &= keep[2];
+        blk.vf[dt].u.w &= keep[3];
       }
     }
 
@@ -174,7 +226,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         for (int r = 0; r < 4; ++r) {
           float x = s[t][n][r] * scale_log2e;
           if (!full) {
-            const int key = key0 + t * 16 + 4 * g + r;
+            const int key = key0 + 8 * g + 4 * t + r;
             const bool vis = key <= qpos[n] && (window <= 0 || key > qpos[n] - window);
             x = vis ? x : -INFINITY;
           }
@@ -207,7 +259,19 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int n = 0; n < NT; ++n)
-        acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
+        acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
+  };
+
+  // two buffers in turn: the next block's loads are in flight while this one is computed
+  Block buf_a, buf_b;
+  if (b0 < b1) load_block(b0, buf_a);
+  for (int kb = b0; kb < b1; kb += 2) {
+    if (kb + 1 < b1) load_block(kb + 1, buf_b);
+    compute(kb, buf_a);
+    if (kb + 1 < b1) {
+      if (kb + 2 < b1) load_block(kb + 2, buf_a);
+      compute(kb + 1, buf_b);
+    }
   }
 
   // ---- finish ---------------------------------------------------------------------------
@@ -303,13 +367,21 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   const int tiles = (int)(((long long)max_q_len * G + rows_per_tile - 1) / rows_per_tile);
   dim3 grid((tiles + 3) / 4, Hk, B * num_splits), block(256);
   const float scale_log2e = scale * 1.4426950408889634f;
-#define GO(NT)                                                                                        \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT>), grid, block, 0, stream, (const bf16_t*)q,     \
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0) {
+    page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+  }
+#define GO(NT, POW2)                                                                                  \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT, POW2>), grid, block, 0, stream, (const bf16_t*)q, \
                      q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
-                     block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, scale_log2e, window,   \
-                     num_splits, part_o, part_ml)
-  if (small) GO(1);
-  else GO(NT_PREFILL);
+                     block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, page_shift,            \
+                     scale_log2e, window, num_splits, part_o, part_ml)
+  const bool pow2 = page_shift >= 3;
+  if (small && pow2) GO(1, true);
+  else if (small) GO(1, false);
+  else if (pow2) GO(NT_PREFILL, true);
+  else GO(NT_PREFILL, false);
 #undef GO
   SA_LAUNCH_CHECK();
   if (num_splits > 1) {

@@ -26,6 +26,8 @@ FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed fp32 instructions stay off on this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core results stay in ordinary vector registers: no moves to and from accumulation registers
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 HEADERS = ["common.h"]
@@ -201,17 +203,20 @@ def compile_many(items: Iterable[Tuple[str, Optional[Dict[str, object]]]], force
     return [r for r in results if r]
 
 
-_loaded: Dict[str, ctypes.CDLL] = {}
+_loaded: Dict[tuple, ctypes.CDLL] = {}
 _load_lock = threading.Lock()
 
 
 def load_library(name: str, defines: Optional[Dict[str, object]] = None, verbose: bool = True) -> ctypes.CDLL:
     """The loaded library, compiled first if no matching build exists."""
-    fn = library_file_name(name, defines)
+    key = (name, tuple(sorted((defines or {}).items())))
+    lib = _loaded.get(key)          # the hot path: no hashing, no lock
+    if lib is not None:
+        return lib
     with _load_lock:
-        lib = _loaded.get(fn)
+        lib = _loaded.get(key)
         if lib is None:
             path = compile_library(name, defines, verbose=verbose)
             lib = ctypes.CDLL(path)
-            _loaded[fn] = lib
+            _loaded[key] = lib
         return lib

@@ -34,20 +34,20 @@ extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, f
 //   v = x[t] + delta[t];  x[t] = v (only when rows == nullptr);  y[r] = v * rsqrt(mean(v^2) + eps) * w
 // rows != nullptr: output row r takes source row rows[r] and x is left untouched.
 // ---------------------------------------------------------------------------------------------
-template <typename TA, typename TW>
-__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TA* __restrict__ delta,
-                                   const TW* __restrict__ w, TA* __restrict__ y,
+template <typename TA, typename TD, typename TW>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int parts,
+                                   size_t part_stride, const TW* __restrict__ w, TA* __restrict__ y,
                                    const int* __restrict__ rows, float eps, int d) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int t = rows ? rows[r] : r;
   float* xr = x + (size_t)t * d;
-  const TA* dr = delta ? delta + (size_t)t * d : nullptr;
+  const TD* dr = delta ? delta + (size_t)t * d : nullptr;
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float v = xr[i];
     if (dr) {
-      v += to_float(dr[i]);
+      for (int p = 0; p < parts; ++p) v += to_float(dr[p * part_stride + i]);
       if (!rows) xr[i] = v;
     }
     ss += v * v;
@@ -57,24 +57,95 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TA* __restrict__
   TA* yr = y + (size_t)r * d;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float v = xr[i];
-    if (dr && rows) v += to_float(dr[i]);
+    if (dr && rows)
+      for (int p = 0; p < parts; ++p) v += to_float(dr[p * part_stride + i]);
     yr[i] = from_float<TA>((v * rs) * to_float(w[i]));
   }
 }
 
-extern "C" int sa_add_rmsnorm(float* x, const void* delta, const void* w, int w_dtype, void* y,
-                              int act_dtype, const int* rows, float eps, int R, int d,
-                              hipStream_t stream) {
+// The same in one pass for d % 4 == 0 and d <= 8192: a thread keeps its (up to 8) groups of four
+// values in registers between the sum of squares and the scaling, and moves 16-byte vectors.
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(bf16_bits_to_float(u.x & 0xffffu), bf16_bits_to_float(u.x >> 16),
+                     bf16_bits_to_float(u.y & 0xffffu), bf16_bits_to_float(u.y >> 16));
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+  uint2 u;
+  u.x = (uint32_t)float_to_bf16_bits(v.x) | ((uint32_t)float_to_bf16_bits(v.y) << 16);
+  u.y = (uint32_t)float_to_bf16_bits(v.z) | ((uint32_t)float_to_bf16_bits(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename TA, typename TD, typename TW>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                              int parts, size_t part_stride,
+                                                              const TW* __restrict__ w, TA* __restrict__ y,
+                                                              const int* __restrict__ rows, float eps, int d) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int t = rows ? rows[r] : r;
+  float* xr = x + (size_t)t * d;
+  const TD* dr = delta ? delta + (size_t)t * d : nullptr;
+  const int groups = d >> 2;
+  float4 v[8], wv[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = (threadIdx.x + k * 256) * 4;
+    if (threadIdx.x + k * 256 < groups) {
+      v[k] = load4(xr + i);
+      wv[k] = load4(w + i);
+      if (dr)
+        for (int p = 0; p < parts; ++p) {
+          const float4 a = load4(dr + p * part_stride + i);
+          v[k].x += a.x; v[k].y += a.y; v[k].z += a.z; v[k].w += a.w;
+        }
+      ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rs = rsqrtf(ss / (float)d + eps);
+  TA* yr = y + (size_t)r * d;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = (threadIdx.x + k * 256) * 4;
+    if (threadIdx.x + k * 256 < groups) {
+      if (dr && !rows) store4(xr + i, v[k]);
+      store4(yr + i, make_float4((v[k].x * rs) * wv[k].x, (v[k].y * rs) * wv[k].y,
+                                 (v[k].z * rs) * wv[k].z, (v[k].w * rs) * wv[k].w));
+    }
+  }
+}
+
+// delta: [T, d] in the activation dtype (delta_dtype == act_dtype, parts == 1), or fp32
+// [parts, T, d] partial sums that are added in order.
+extern "C" int sa_add_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const void* w,
+                              int w_dtype, void* y, int act_dtype, const int* rows, float eps, int R,
+                              int T, int d, hipStream_t stream) {
   if (R <= 0) return 0;
-  if (d <= 0) return SA_ERR_ARG;
-  dim3 grid(R), block(d >= 1024 ? 256 : 64);
-#define GO(TA, TW)                                                                                \
-  hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TW>), grid, block, 0, stream, x, (const TA*)delta,  \
-                     (const TW*)w, (TA*)y, rows, eps, d)
-  if (act_dtype == SA_F32 && w_dtype == SA_F32) GO(float, float);
-  else if (act_dtype == SA_F32 && w_dtype == SA_BF16) GO(float, bf16_t);
-  else if (act_dtype == SA_BF16 && w_dtype == SA_F32) GO(bf16_t, float);
-  else if (act_dtype == SA_BF16 && w_dtype == SA_BF16) GO(bf16_t, bf16_t);
+  if (d <= 0 || parts < 1) return SA_ERR_ARG;
+  if (delta && delta_dtype != act_dtype && delta_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
+  if (delta && parts > 1 && delta_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
+  const size_t part_stride = (size_t)T * d;
+  const bool vec = (d & 3) == 0 && d <= 8192 && d >= 256;
+  dim3 grid(R), block(vec || d >= 1024 ? 256 : 64);
+#define GO(TA, TD, TW)                                                                                   \
+  do {                                                                                                   \
+    if (vec)                                                                                             \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TD, TW>), grid, block, 0, stream, x,                \
+                         (const TD*)delta, parts, part_stride, (const TW*)w, (TA*)y, rows, eps, d);      \
+    else                                                                                                 \
+      hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TD, TW>), grid, block, 0, stream, x, (const TD*)delta,  \
+                         parts, part_stride, (const TW*)w, (TA*)y, rows, eps, d);                        \
+  } while (0)
+  const bool dfloat = delta && delta_dtype == SA_F32;
+  if (act_dtype == SA_F32 && w_dtype == SA_F32) GO(float, float, float);
+  else if (act_dtype == SA_F32 && w_dtype == SA_BF16) GO(float, float, bf16_t);
+  else if (act_dtype == SA_BF16 && w_dtype == SA_F32) { if (dfloat) GO(bf16_t, float, float); else GO(bf16_t, bf16_t, float); }
+  else if (act_dtype == SA_BF16 && w_dtype == SA_BF16) { if (dfloat) GO(bf16_t, float, bf16_t); else GO(bf16_t, bf16_t, bf16_t); }
   else return SA_ERR_UNSUPPORTED;
 #undef GO
   SA_LAUNCH_CHECK();

@@ -23,9 +23,10 @@ union Frag {
   bf16x8_t v;
 };
 
-#define KU 4  // k-chunks of 32 loaded before their products are issued
-
-template <int RT, int MT, int KS, typename TC, bool SWIGLU>
+// KU = k-chunks of 32 loaded before their products are issued (loads in flight per wave).
+// gridDim.z > 1 cuts K across workgroups as well: workgroup z writes its partial sums to
+// C + z * M * N (fp32), and the consumer adds the parts in order.
+template <int RT, int MT, int KS, int KU, typename TC, bool SWIGLU>
 __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                              const bf16_t* __restrict__ W,
                                                              TC* __restrict__ C, int M, int N, int K,
@@ -42,9 +43,13 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   const int m0 = blockIdx.y * (MT * 16);
 
   const int nchunks = (K + 31) >> 5;
-  const int per = (nchunks + KS - 1) / KS;
-  const int ch_begin = wave * per;
-  const int ch_end = min(nchunks, ch_begin + per);
+  const int per_wg = (nchunks + gridDim.z - 1) / gridDim.z;
+  const int wg_begin = blockIdx.z * per_wg;
+  const int wg_end = min(nchunks, wg_begin + per_wg);
+  const int per = (per_wg + KS - 1) / KS;
+  const int ch_begin = wg_begin + wave * per;
+  const int ch_end = min(wg_end, ch_begin + per);
+  C += (size_t)blockIdx.z * M * N;
 
   const bf16_t* wrow[RT];
   bool wok[RT];
@@ -147,12 +152,12 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   }
 }
 
-template <int RT, int MT, int KS, typename TC, bool SWIGLU>
+template <int RT, int MT, int KS, int KU, typename TC, bool SWIGLU>
 static int launch_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
-                         hipStream_t stream) {
-  dim3 grid((N + (SWIGLU ? 16 : RT * 16) - 1) / (SWIGLU ? 16 : RT * 16), (M + MT * 16 - 1) / (MT * 16));
-  if (grid.y > 65535) return SA_ERR_ARG;
-  hipLaunchKernelGGL((gemm_skinny_kernel<RT, MT, KS, TC, SWIGLU>), grid, dim3(64 * KS), 0, stream,
+                         int parts, hipStream_t stream) {
+  dim3 grid((N + (SWIGLU ? 16 : RT * 16) - 1) / (SWIGLU ? 16 : RT * 16), (M + MT * 16 - 1) / (MT * 16), parts);
+  if (grid.y > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, MT, KS, KU, TC, SWIGLU>), grid, dim3(64 * KS), 0, stream,
                      (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, up_offset);
   SA_LAUNCH_CHECK();
   return 0;
@@ -160,34 +165,42 @@ static int launch_skinny(const void* A, const void* W, void* C, int M, int N, in
 
 template <typename TC, bool SWIGLU>
 static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
-                       hipStream_t stream) {
+                       int parts, hipStream_t stream) {
   // rows of activations per workgroup: 16, 32 or 64 (larger M loops over grid.y)
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  // many weight rows: 2 row tiles per wave and 4 waves; few rows: 1 tile and 16 waves splitting K
+  // many weight rows: 2 row tiles per wave and 4 waves; few rows: 1 tile and more waves splitting K
   const bool wide = SWIGLU || N >= 8192;
-#define GO(RT, MT, KS) return launch_skinny<RT, MT, KS, TC, SWIGLU>(A, W, C, M, N, K, up_offset, stream)
+#define GO(RT, MT, KS, KU) \
+  return launch_skinny<RT, MT, KS, KU, TC, SWIGLU>(A, W, C, M, N, K, up_offset, parts, stream)
   if (wide) {
-    if (mt == 1) GO(2, 1, 4);
-    if (mt == 2) GO(2, 2, 4);
-    GO(2, 4, 4);
+    if (mt == 1) GO(2, 1, 4, 8);
+    if (mt == 2) GO(2, 2, 4, 4);
+    GO(2, 4, 4, 4);
   }
   if constexpr (!SWIGLU) {
+    if (parts > 1) {
+      // K is already cut across workgroups: 4 waves each
+      if (mt == 1) GO(1, 1, 4, 8);
+      if (mt == 2) GO(1, 2, 4, 4);
+      GO(1, 4, 4, 4);
+    }
     // 16 waves leave 128 registers a lane, enough only for one activation tile
-    if (mt == 1) GO(1, 1, 16);
-    if (mt == 2) GO(1, 2, 8);
-    GO(1, 4, 8);
+    if (mt == 1) GO(1, 1, 16, 4);
+    if (mt == 2) GO(1, 2, 8, 4);
+    GO(1, 4, 8, 4);
   }
 #undef GO
   return SA_ERR_ARG;
 }
 
-// C = A W^T; c_dtype SA_BF16 or SA_F32
+// C = A W^T; c_dtype SA_BF16 or SA_F32.  parts > 1 (fp32 only): C is [parts, M, N] and holds
+// partial sums over `parts` slices of K, to be added by the consumer.
 extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K,
-                                   hipStream_t stream) {
+                                   int parts, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || (K & 7)) return SA_ERR_ARG;
-  if (c_dtype == SA_BF16) return pick_skinny<bf16_t, false>(A, W, C, M, N, K, 0, stream);
-  if (c_dtype == SA_F32) return pick_skinny<float, false>(A, W, C, M, N, K, 0, stream);
+  if (K <= 0 || (K & 7) || parts < 1) return SA_ERR_ARG;
+  if (c_dtype == SA_BF16 && parts == 1) return pick_skinny<bf16_t, false>(A, W, C, M, N, K, 0, 1, stream);
+  if (c_dtype == SA_F32) return pick_skinny<float, false>(A, W, C, M, N, K, 0, parts, stream);
   return SA_ERR_UNSUPPORTED;
 }
 
@@ -196,5 +209,5 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
                                           hipStream_t stream) {
   if (M <= 0 || I <= 0) return 0;
   if (K <= 0 || (K & 7)) return SA_ERR_ARG;
-  return pick_skinny<bf16_t, true>(A, W, C, M, I, K, I, stream);
+  return pick_skinny<bf16_t, true>(A, W, C, M, I, K, I, 1, stream);
 }

@@ -89,6 +89,8 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x += delta (fp32 residual stream, in place), out = rmsnorm(x) * weight.
 
+    `delta` is [T, d] in the activation dtype or fp32, or fp32 [parts, T, d]: partial sums of a
+    product whose inner dimension was cut across workgroups; the parts are added in order.
     With `rows`, only the listed rows are produced (out[r] from source row rows[r]) and x is
     left as it was."""
     _dev(x, delta, weight, out, rows)
@@ -99,12 +101,19 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     if rows is not None:
         _i32(rows, R, "rows")
     _check(out.shape == (R, d), f"norm output must be [{R}, {d}]")
+    parts, delta_code = 1, _code(out)
     if delta is not None:
-        _check(delta.shape == (T, d) and delta.dtype == out.dtype, "delta must be [T, d] in the activation dtype")
+        if delta.dim() == 3:
+            parts = delta.shape[0]
+            _check(delta.dtype == torch.float32 and delta.shape[1:] == (T, d), "partial deltas must be fp32 [parts, T, d]")
+        else:
+            _check(delta.shape == (T, d) and delta.dtype in (out.dtype, torch.float32),
+                   "delta must be [T, d] in the activation dtype or fp32")
+        delta_code = _code(delta)
     lib = load_library("elementwise")
-    _ret(lib.sa_add_rmsnorm(_ptr(x), _ptr(delta), _ptr(weight), c_int(_code(weight)), _ptr(out),
-                            c_int(_code(out)), _ptr(rows), c_float(eps), c_int(R), c_int(d), _stream()),
-         "add_rmsnorm")
+    _ret(lib.sa_add_rmsnorm(_ptr(x), _ptr(delta), c_int(delta_code), c_int(parts), _ptr(weight),
+                            c_int(_code(weight)), _ptr(out), c_int(_code(out)), _ptr(rows), c_float(eps),
+                            c_int(R), c_int(T), c_int(d), _stream()), "add_rmsnorm")
     return out
 
 
@@ -235,16 +244,38 @@ def mfma_gemm_available(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> 
 
 
 def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out = a @ w^T on the matrix cores, weights streamed once per 64 rows of a."""
+    """out = a @ w^T on the matrix cores, weights streamed once per 64 rows of a.
+
+    `out` [M, N] bf16 or fp32; or fp32 [parts, M, N]: the inner dimension is cut into `parts`
+    slices over workgroups and slice p's partial sums go to out[p] (the consumer adds them)."""
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
-    _check(w.shape == (N, K) and out.shape == (M, N), "gemm_bf16_skinny: shapes do not match")
+    parts = 1
+    if out.dim() == 3:
+        parts = out.shape[0]
+        _check(out.dtype == torch.float32 and out.shape[1:] == (M, N), "partial sums must be fp32 [parts, M, N]")
+    else:
+        _check(out.shape == (M, N), "gemm_bf16_skinny: shapes do not match")
+    _check(w.shape == (N, K), "gemm_bf16_skinny: shapes do not match")
     _check(mfma_gemm_available(a, w, out), "gemm_bf16_skinny needs bf16 operands, K % 8 == 0 and 16-byte alignment")
     lib = load_library("gemm_mfma")
     _ret(lib.sa_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), c_int(_code(out)), c_int(M), c_int(N), c_int(K),
-                                 _stream()), "gemm_bf16_skinny")
+                                 c_int(parts), _stream()), "gemm_bf16_skinny")
     return out
+
+
+def split_k_parts(M: int, N: int, K: int) -> int:
+    """Into how many slices the inner dimension of a few-row product is cut across workgroups so
+    that a matrix with few rows still fills the chip (about 512 workgroups, slices of at least
+    256): 1 means no cut."""
+    if M > 16 or N >= 8192:
+        return 1
+    tiles = -(-N // 16)
+    parts = 1
+    while parts < 8 and tiles * parts < 512 and K // (parts * 2) >= 256:
+        parts *= 2
+    return parts
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -9,6 +9,7 @@ Roles and what each must offer:
 * norm          `forward(x, delta, rows=None) -> y`: adds `delta` (or nothing) into the fp32
                 residual stream `x` in place and returns the normalised activations in the
                 activation dtype; with `rows` it returns only those rows and leaves x alone.
+                `delta` is [T, d], or fp32 [parts, T, d] partial sums to be added in order.
 * position      owned by a mixer; `apply(...)` as the mixer needs it (the rotary part rotates q
                 and k while k and v are written to the cache).
 * mixer         `forward(h, ctx, cache, writes_cache) -> delta [T, d]`; may ask for per-token

@@ -18,9 +18,19 @@ from .. import ops
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+           out: Optional[torch.Tensor] = None, partial_ok: bool = False) -> torch.Tensor:
+    """a @ w^T.  With `partial_ok` the result may be fp32 [parts, M, N] partial sums (see
+    `ops.gemm_bf16_skinny`): for callers whose consumer adds the parts, as the norms do."""
     M = a.shape[0]
     N = w.shape[0]
+    if (partial_ok and out is None and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and 0 < M <= ops.SKINNY_MAX_ROWS):
+        # few rows: the product stays fp32 on its way into the residual stream, in one or more parts
+        parts = ops.split_k_parts(M, N, a.shape[1])
+        out = torch.empty((parts, M, N), dtype=torch.float32, device=a.device)
+        if ops.mfma_gemm_available(a, w, out):
+            return ops.gemm_bf16_skinny(a, w, out)
+        out = None
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
     if M == 0:

@@ -152,7 +152,7 @@ class GQAAttention(Part):
         attn = self.rt.empty((T, self.num_heads * self.head_dim))
         ops.paged_attention(qkv, qkv.shape[1], attn, cache.k_pages, cache.v_pages, grp.block_table, ctx,
                             self.num_heads, self.scale, self.window)
-        return linear(attn, self.wo)
+        return linear(attn, self.wo, partial_ok=True)      # the following norm adds the parts
 
 
 # ---------------------------------------------------------------------------------------------
@@ -187,7 +187,7 @@ class SwiGLU(Part):
         else:
             gu = linear(h, self.w_gate_up)
             ops.silu_mul(gu, a)
-        return linear(a, self.w_down)
+        return linear(a, self.w_down, partial_ok=True)     # the following norm adds the parts
 
 
 # ---------------------------------------------------------------------------------------------

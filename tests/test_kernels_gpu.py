@@ -407,3 +407,27 @@ def test_kernels_refuse_what_they_do_not_take():
                                    torch.tensor([0, 1], dtype=torch.int32, device=DEV),
                                    torch.tensor([1], dtype=torch.int32, device=DEV),
                                    torch.zeros(1, dtype=torch.int32, device=DEV), 1, 1, 1.0, None)
+
+
+@pytest.mark.parametrize("M,N,K,parts", [(1, 2048, 2048, 4), (8, 2048, 8192, 2), (16, 96, 256, 8), (5, 77, 520, 3)])
+def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
+    from serve_amd import ops
+    a = rnd((M, K), torch.bfloat16, 4)
+    w = rnd((N, K), torch.bfloat16, 5, 0.05)
+    out = torch.empty((parts, M, N), dtype=torch.float32, device=DEV)
+    ops.gemm_bf16_skinny(a, w, out)
+    want = a.double() @ w.double().T
+    torch.testing.assert_close(out.double().sum(0), want, atol=2e-4 * K ** 0.5, rtol=1e-4)
+    assert out[0].abs().max() > 0 and not torch.allclose(out[0].double(), want)       # really parts
+    # the norm adds the parts into the residual stream in order
+    x = rnd((M, N), torch.float32, 6)
+    x0 = x.clone()
+    g = rnd((N,), torch.bfloat16, 7) * 0.1 + 1
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(x, out, g, 1e-5, y)
+    xs = x0.double() + want
+    torch.testing.assert_close(x.double(), xs, atol=1e-3, rtol=1e-4)
+    ref = xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + 1e-5) * g.double()
+    torch.testing.assert_close(y.double(), ref, atol=2e-2, rtol=1e-2)
+    assert ops.split_k_parts(8, 2048, 2048) > 1 and ops.split_k_parts(8, 16384, 2048) == 1
+    assert ops.split_k_parts(64, 2048, 2048) == 1

@@ -87,8 +87,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int kb_lo = lo_key >> 5;
   const int kb_hi = hi_key >> 5;
   const int per = (kb_hi - kb_lo + num_splits) / num_splits;   // ceil((kb_hi - kb_lo + 1) / splits)
-  const int b0 = kb_lo + sp * per;
-  const int b1 = min(kb_hi + 1, b0 + per);
+  // the same for every lane: say so, or the integer division makes the whole loop control vector work
+  const int b0 = __builtin_amdgcn_readfirstlane(kb_lo + sp * per);
+  const int b1 = __builtin_amdgcn_readfirstlane(min(kb_hi + 1, b0 + per));
   const int* bt = block_table + (size_t)seg * max_pages;
 
   // this lane's query column in each column tile
@@ -132,25 +133,47 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     Frag kf[2][DC];
     Frag vf[DT];
   };
-  // key index -> (page, offset in the page); a shift when the page size is a power of two
-  auto locate = [&](int key, int& page, int& off) {
-    int idx;
+  // Page ids.  With a power-of-two page size a block of 32 keys spans at most four pages, the
+  // same for every lane: they are fetched with scalar loads one block ahead (`pgn`), which keeps
+  // them out of the vector-memory queue, so that waiting for them does not drain the K/V loads.
+  const int last_idx = POW2 ? ((ctx - 1) >> page_shift) : 0;
+  const int ppb_shift = POW2 ? page_shift : 0;
+  int pgn[4] = {0, 0, 0, 0};
+  auto prefetch_pages = [&](int kb) {
     if (POW2) {
-      idx = key >> page_shift;
-      off = key & (page_size - 1);
-    } else {
-      idx = key / page_size;
-      off = key - idx * page_size;
+      const int first = (kb << 5) >> ppb_shift;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = __builtin_amdgcn_readfirstlane(min(first + j, last_idx));
+        pgn[j] = __builtin_amdgcn_readfirstlane(max(bt[idx], 0));
+      }
     }
+  };
+  auto pick = [&](const int (&pg)[4], int j) {          // two-level select, no branches
+    const int lo = (j & 1) ? pg[1] : pg[0];
+    const int hi = (j & 1) ? pg[3] : pg[2];
+    return (j & 2) ? hi : lo;
+  };
+  // key index -> (page, offset in the page) for page sizes that are no power of two
+  auto locate = [&](int key, int& page, int& off) {
+    const int idx = key / page_size;
+    off = key - idx * page_size;
     page = max(bt[idx], 0);
   };
   auto load_block = [&](int kb, Block& blk) {
     const int key0 = kb << 5;
+    int pg[4] = {pgn[0], pgn[1], pgn[2], pgn[3]};
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int kk = min(key0 + 8 * (c >> 2) + 4 * t + (c & 3), ctx - 1);
+      const int ko = 8 * (c >> 2) + 4 * t + (c & 3);
+      const int kk = min(key0 + ko, ctx - 1);
       int page, off;
-      locate(kk, page, off);
+      if (POW2) {
+        page = pick(pg, page_shift >= 5 ? 0 : (ko >> page_shift));
+        off = kk & (page_size - 1);
+      } else {
+        locate(kk, page, off);
+      }
       const bf16_t* kp = k_pages + (size_t)page * k_page_stride + ((size_t)hk * page_size + off) * HD;
 #pragma unroll
       for (int dc = 0; dc < DC; ++dc) {
@@ -160,8 +183,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
     if (wide_v) {
       const int run = min(key0 + 8 * g, (ctx - 1) & ~7);
-      int page, off;
-      locate(run, page, off);
+      const int page = pick(pg, page_shift >= 5 ? 0 : ((8 * g) >> page_shift));
+      const int off = run & (page_size - 1);
       const bf16_t* vp = v_pages + (size_t)page * k_page_stride + (size_t)hk * HD * page_size + off;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
@@ -178,6 +201,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
           blk.vf[dt].h[h] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * page_size);
       }
     }
+    prefetch_pages(kb + 1);
   };
 
   auto compute = [&](int kb, Block& blk) {
@@ -262,15 +286,21 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
   };
 
-  // two buffers in turn: the next block's loads are in flight while this one is computed
-  Block buf_a, buf_b;
+  // three buffers in turn: the loads of the next two blocks are in flight while one is computed
+  Block buf_a, buf_b, buf_c;
+  prefetch_pages(b0);
   if (b0 < b1) load_block(b0, buf_a);
-  for (int kb = b0; kb < b1; kb += 2) {
-    if (kb + 1 < b1) load_block(kb + 1, buf_b);
+  if (b0 + 1 < b1) load_block(b0 + 1, buf_b);
+  for (int kb = b0; kb < b1; kb += 3) {
+    if (kb + 2 < b1) load_block(kb + 2, buf_c);
     compute(kb, buf_a);
     if (kb + 1 < b1) {
-      if (kb + 2 < b1) load_block(kb + 2, buf_a);
+      if (kb + 3 < b1) load_block(kb + 3, buf_a);
       compute(kb + 1, buf_b);
+    }
+    if (kb + 2 < b1) {
+      if (kb + 4 < b1) load_block(kb + 4, buf_b);
+      compute(kb + 2, buf_c);
     }
   }
 

@@ -26,7 +26,8 @@ union Frag {
 // KU = k-chunks of 32 loaded before their products are issued (loads in flight per wave).
 // gridDim.z > 1 cuts K across workgroups as well: workgroup z writes its partial sums to
 // C + z * M * N (fp32), and the consumer adds the parts in order.
-template <int RT, int MT, int KS, int KU, typename TC, bool SWIGLU>
+// STREAM: weights are loaded with the non-temporal hint (they are read once per step).
+template <int RT, int MT, int KS, int KU, typename TC, bool SWIGLU, bool STREAM = false>
 __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                              const bf16_t* __restrict__ W,
                                                              TC* __restrict__ C, int M, int N, int K,
@@ -86,7 +87,16 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         wf[rt][u].u = zero;
-        if (kin && wok[rt]) wf[rt][u].u = *reinterpret_cast<const uint4*>(wrow[rt] + k);
+        if (kin && wok[rt]) {
+          const uint4* src = reinterpret_cast<const uint4*>(wrow[rt] + k);
+          if (STREAM) {
+            typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+            const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
+            wf[rt][u].u = make_uint4(t.x, t.y, t.z, t.w);
+          } else {
+            wf[rt][u].u = *src;
+          }
+        }
       }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
@@ -172,15 +182,16 @@ static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int 
   const bool wide = SWIGLU || N >= 8192;
 #define GO(RT, MT, KS, KU) \
   return launch_skinny<RT, MT, KS, KU, TC, SWIGLU>(A, W, C, M, N, K, up_offset, parts, stream)
+  // (the choices below are the best of a sweep over RT, KS and KU at the Llama-3.2-1B sizes)
   if (wide) {
-    if (mt == 1) GO(2, 1, 4, 8);
+    if (mt == 1) GO(2, 1, 2, 8);
     if (mt == 2) GO(2, 2, 4, 4);
     GO(2, 4, 4, 4);
   }
   if constexpr (!SWIGLU) {
     if (parts > 1) {
-      // K is already cut across workgroups: 4 waves each
-      if (mt == 1) GO(1, 1, 4, 8);
+      // K is already cut across workgroups: 2 waves each
+      if (mt == 1) GO(1, 1, 2, 8);
       if (mt == 2) GO(1, 2, 4, 4);
       GO(1, 4, 4, 4);
     }

@@ -273,7 +273,7 @@ def split_k_parts(M: int, N: int, K: int) -> int:
         return 1
     tiles = -(-N // 16)
     parts = 1
-    while parts < 8 and tiles * parts < 512 and K // (parts * 2) >= 256:
+    while parts < 8 and tiles * parts < 1024 and K // (parts * 2) >= 512:
         parts *= 2
     return parts
 

@@ -30,6 +30,9 @@ class EngineConfig:
     device: str = "cuda:0"
     # replay a decode-only step from a captured HIP graph
     use_graphs: bool = True
+    # launch a decode step before the previous step's tokens have reached the host (they are fed
+    # back on the device); needs graphs, no stop tokens and nobody keeping logits
+    async_decode: bool = True
 
     def validate(self) -> None:
         if self.dtype not in DTYPES:

@@ -6,23 +6,31 @@
 // ---------------------------------------------------------------------------------------------
 // embedding: x[t, :] = table[tokens[t], :]   (serve/model.py:220), residual stream in fp32
 // ---------------------------------------------------------------------------------------------
+// A token id comes from `tokens[t]`, or, when src_row[t] >= 0, from prev[src_row[t]]: the token
+// that an earlier step sampled on the device and that the host has not read back yet.
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ x, int d) {
+                             const int* __restrict__ src_row, const int* __restrict__ prev,
+                             float* __restrict__ x, int d, int V) {
   const int t = blockIdx.x;
-  const size_t row = (size_t)tokens[t] * (size_t)d;
+  int tok = tokens[t];
+  if (src_row && src_row[t] >= 0) tok = prev[src_row[t]];
+  tok = min(max(tok, 0), V - 1);
+  const size_t row = (size_t)tok * (size_t)d;
   for (int i = threadIdx.x; i < d; i += blockDim.x) x[(size_t)t * d + i] = to_float(table[row + i]);
 }
 
-extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, float* x, int T, int d,
-                        hipStream_t stream) {
+extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, const int* src_row,
+                        const int* prev, float* x, int T, int d, int V, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (d <= 0) return SA_ERR_ARG;
+  if (d <= 0 || V <= 0 || (src_row && !prev)) return SA_ERR_ARG;
   dim3 grid(T), block(256);
   if (table_dtype == SA_F32)
-    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, x, d);
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, src_row, prev,
+                       x, d, V);
   else if (table_dtype == SA_BF16)
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, x, d);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, src_row, prev,
+                       x, d, V);
   else
     return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();

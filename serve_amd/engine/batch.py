@@ -59,6 +59,9 @@ class StepContext:
     max_ctx_len: int = 0
     max_pages: int = 0
     decode_only: bool = False
+    # decode steps replayed from a graph: rows whose token comes from the device (see runner)
+    src_row: Optional[torch.Tensor] = None
+    prev_tokens: Optional[torch.Tensor] = None
 
 
 def _align(n: int) -> int:

@@ -9,7 +9,10 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
+
+from .. import ops
 
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage, bytes_per_page, group_windows
@@ -23,14 +26,41 @@ GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
 
 class _GraphEntry:
-    def __init__(self, layout: StepLayout, device: torch.device):
-        self.layout = layout
-        self.stage = torch.zeros(layout.total, dtype=torch.int32).pin_memory()
-        self.device_buf = torch.zeros(layout.total, dtype=torch.int32, device=device)
+    """Fixed buffers and the captured graph of decode-only steps of one shape."""
+
+    def __init__(self, b_pad: int, max_pages: int, num_groups: int, device: torch.device):
+        self.b_pad = b_pad
+        self.layout = StepLayout(b_pad, b_pad, b_pad, max_pages, num_groups)
+        # after the step's index arrays: where each row's token comes from, and the sampling inputs
+        o = self.layout.total
+        self.off_src_row = o
+        self.off_temps = o + _pad4(b_pad)
+        self.off_keys = o + 2 * _pad4(b_pad)
+        self.total = o + 2 * _pad4(b_pad) + _pad4(2 * b_pad)
+        self.stage = torch.zeros(self.total, dtype=torch.int32).pin_memory()
+        self.device_buf = torch.zeros(self.total, dtype=torch.int32, device=device)
+        self.host_tokens = [torch.zeros(b_pad, dtype=torch.int32).pin_memory() for _ in range(2)]
         self.copied = torch.cuda.Event()
         self.graph = None
         self.logits = None
         self.runs = 0
+        self.launches = 0
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class DecodeHandle:
+    """A launched decode step whose sampled tokens have not been read back yet."""
+
+    def __init__(self, host_tokens: torch.Tensor, event, n: int):
+        self.host_tokens, self.event, self.n = host_tokens, event, n
+
+    def tokens(self) -> List[int]:
+        self.event.synchronize()
+        return self.host_tokens[: self.n].tolist()
+
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -70,6 +100,9 @@ class ModelRunner:
                                   cfg.max_pages_per_request)
         self.storage = CacheStorage(rt, creq, sreq, self.windows, num_pages, cfg.page_size, cfg.max_requests)
         self._graphs = {}
+        # tokens sampled by the latest decode launch, by row: the next launch may read them here
+        self.sampled = torch.zeros(GRAPH_BATCHES[-1], dtype=torch.int32, device=rt.device)
+        self._row_of = {}
         self._use_graphs = bool(cfg.use_graphs) and model.graph_safe()
 
     # -- requests -------------------------------------------------------------------------------
@@ -106,60 +139,106 @@ class ModelRunner:
         return logits
 
     # -- decode-only steps replayed from HIP graphs ---------------------------------------------------
-    def _decode_step(self, segments: Sequence[Segment]):
-        """One token per request.  The kernel sequence of such a step depends only on the padded
-        batch size and on the bucket of the longest context (which fixes the attention's key
-        splits), so it is captured once per (batch, bucket) into a HIP graph and replayed: the
-        step's index arrays are copied into the graph's fixed buffer, everything else is one
-        launch.  The first step of a shape runs eagerly and is then captured."""
+    def _decode_core(self, segments: Sequence[Segment], temps=None, keys=None, src_rows=None):
+        """One token per request, sampling included.  The kernel sequence of such a step depends
+        only on the padded batch size and on the bucket of the longest context (which fixes the
+        attention's key splits), so it is captured once per (batch, bucket) into a HIP graph and
+        replayed: the step's index arrays are copied into the graph's fixed buffer, everything
+        else is one launch.  The first two steps of a shape run eagerly, then it is captured.
+
+        A row's token id is given by the caller, or (src_rows[i] >= 0) is the token that the
+        previous launch sampled into row src_rows[i] of `self.sampled` and that never left the
+        device.  Returns (entry, logits, context lengths)."""
         B = len(segments)
         b_pad = next(b for b in GRAPH_BATCHES if b >= B)
         mp = self.cfg.max_pages_per_request
         lay, host, facts = plan_step(segments, self.cache, self.vocab_size, pad_segments_to=b_pad,
                                      fixed_max_pages=mp)
-        # all rows' logits are computed; the wanted ones are picked afterwards
-        wanted = host[lay.logit_rows: lay.logit_rows + lay.R].copy()
         bucket = 256
         while bucket < facts["max_ctx_len"]:
             bucket *= 2
         key = (b_pad, bucket)
         entry = self._graphs.get(key)
         if entry is None:
-            entry = self._graphs[key] = _GraphEntry(StepLayout(b_pad, b_pad, b_pad, mp, self.cache.num_groups),
-                                                    self.rt.device)
+            entry = self._graphs[key] = _GraphEntry(b_pad, mp, self.cache.num_groups, self.rt.device)
         full = entry.layout
-        stage = entry.stage
         entry.copied.synchronize()          # the previous step's copy out of the staging buffer is done
-        stage.zero_()
-        sn = stage.numpy()
+        sn = entry.stage.numpy()
+        sn[:] = 0
         for name in ("token_ids", "positions", "seg_of_token", "cu_q", "ctx_len", "state_slots"):
             a, b = getattr(lay, name), getattr(full, name)
             n = {"cu_q": b_pad + 1}.get(name, b_pad)
             sn[b: b + n] = host[a: a + n]
-        sn[full.logit_rows: full.logit_rows + b_pad] = range(b_pad)
+        sn[full.logit_rows: full.logit_rows + b_pad] = range(b_pad)     # every row's logits are computed
         for g in range(self.cache.num_groups):
             sn[full.block_tables[g]: full.block_tables[g] + b_pad * mp] = \
                 host[lay.block_tables[g]: lay.block_tables[g] + b_pad * mp]
             sn[full.slots[g]: full.slots[g] + b_pad] = host[lay.slots[g]: lay.slots[g] + b_pad]
-        entry.device_buf.copy_(stage, non_blocking=True)
+        sn[entry.off_src_row: entry.off_src_row + b_pad] = -1
+        if src_rows is not None:
+            sn[entry.off_src_row: entry.off_src_row + B] = src_rows
+        if temps is not None:
+            sn[entry.off_temps: entry.off_temps + B].view(np.float32)[:] = temps
+            sn[entry.off_keys: entry.off_keys + 2 * B].view(np.int64)[:] = keys
+        entry.device_buf.copy_(entry.stage, non_blocking=True)
         entry.copied.record()
         if entry.graph is None:
             facts = dict(facts, max_ctx_len=bucket)
             ctx = context_from(full, entry.device_buf, facts)
+            ctx.src_row = entry.device_buf[entry.off_src_row: entry.off_src_row + b_pad]
+            ctx.prev_tokens = self.sampled
+            t_dev = entry.device_buf[entry.off_temps: entry.off_temps + b_pad].view(torch.float32)
+            k_dev = entry.device_buf[entry.off_keys: entry.off_keys + 2 * b_pad].view(torch.int64)
+
+            def run():
+                logits = self.model.forward(ctx, self.storage.layers)
+                ops.sample(logits, t_dev, k_dev, self.sampled[:b_pad])
+                return logits
             entry.runs += 1
-            logits = self.model.forward(ctx, self.storage.layers)
+            logits = run()
             if entry.runs >= 2:
                 # every library is loaded and warm by now: capture for the following steps
                 g = torch.cuda.CUDAGraph()
                 torch.cuda.synchronize()
                 with torch.cuda.graph(g):
-                    entry.logits = self.model.forward(ctx, self.storage.layers)
+                    entry.logits = run()
                 entry.graph = g
         else:
             entry.graph.replay()
             logits = entry.logits
-        if len(wanted) == B:
-            logits = logits[:B]
+        return entry, logits, facts["ctx_lens"][:B]
+
+    def _decode_step(self, segments: Sequence[Segment]):
+        entry, logits, ctx_lens = self._decode_core(segments)
+        wanted = [i for i, s in enumerate(segments) if len(s.want)]
+        if len(wanted) == len(segments):
+            logits = logits[: len(segments)]
         else:
             logits = logits[torch.as_tensor(wanted, dtype=torch.long, device=logits.device)]
-        return logits, facts["ctx_lens"][:B]
+        return logits, ctx_lens
+
+    def can_decode_async(self, n: int) -> bool:
+        return self._use_graphs and 0 < n <= GRAPH_BATCHES[-1]
+
+    @torch.inference_mode()
+    def decode_launch(self, req_ids: Sequence, tokens: Sequence[Optional[int]], temperatures: Sequence[float],
+                      keys: Sequence[int]) -> DecodeHandle:
+        """Launch one decode step for the given requests, sampling on the device, and return at
+        once.  tokens[i] is request i's token, or None for "the token that the previous launch
+        sampled for this request" (it is taken on the device; every request of that launch's
+        tokens is still in `self.sampled`).  `keys` are the sampling keys of the rows
+        (`serve_amd.sampling.sampler.row_key`); rows with temperature 0 are greedy."""
+        with torch.cuda.device(self.rt.device):
+            src = [-1 if t is not None else self._row_of[r] for r, t in zip(req_ids, tokens)]
+            segments = [Segment(r, [0 if t is None else t], [0]) for r, t in zip(req_ids, tokens)]
+            entry, _, ctx_lens = self._decode_core(segments, np.asarray(temperatures, dtype=np.float32),
+                                                   np.asarray(keys, dtype=np.int64), src)
+            self._row_of = {r: i for i, r in enumerate(req_ids)}
+            host = entry.host_tokens[entry.launches & 1]
+            entry.launches += 1
+            host.copy_(self.sampled[: entry.b_pad], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+        for r, n in zip(req_ids, ctx_lens):
+            self.cache.trim(r, n)
+        return DecodeHandle(host, ev, len(req_ids))

@@ -47,6 +47,15 @@ class GenerationRequest:
     def all_tokens(self) -> List[int]:
         return self.prompt + self.generated
 
+    def tokens_between(self, a: int, b: int) -> List[int]:
+        """Tokens a..b-1 of prompt + generated, without joining the two lists."""
+        n = len(self.prompt)
+        if b <= n:
+            return self.prompt[a:b]
+        if a >= n:
+            return self.generated[a - n: b - n]
+        return self.prompt[a:] + self.generated[: b - n]
+
     def pending(self) -> int:
         return len(self.prompt) + len(self.generated) - self.fed
 
@@ -80,6 +89,10 @@ class Scheduler:
         self._reservation = {}
         self.steps = 0
         self.step_log: List[dict] = []       # one record per step, for tests and tracing
+        # decode steps whose tokens are still on the device: the host runs one step ahead
+        self._inflight = None
+        self.async_decode = (bool(getattr(cfg, "async_decode", True)) and hasattr(runner, "decode_launch")
+                             and hasattr(sampler, "seed") and not self.eos)
 
     # -- life cycle of a request ----------------------------------------------------------------
     def _total_pages(self, g: int) -> int:
@@ -98,6 +111,7 @@ class Scheduler:
         self.finished.append(r)
 
     def _preempt(self, r: GenerationRequest) -> None:
+        self._resolve()                       # its generated tokens become part of its new prompt
         self.runner.release(r.req_id)
         self.running.remove(r)
         r.fed = 0
@@ -242,11 +256,15 @@ class Scheduler:
         """Plan and run one step.  False when nothing is left to do."""
         plan = self.plan()
         if not plan.requests:
+            self._resolve()
             return False
+        if self._pipelinable(plan):
+            self._launch_decode(plan)
+            return True
+        self._resolve()                       # the tokens of the step in flight are needed on the host
         segments = []
         for r, n, s in zip(plan.requests, plan.counts, plan.samples):
-            toks = r.all_tokens()[r.fed: r.fed + n]
-            segments.append(Segment(r.req_id, toks, [n - 1] if s else []))
+            segments.append(Segment(r.req_id, r.tokens_between(r.fed, r.fed + n), [n - 1] if s else []))
         logits = self.runner.step(segments, borrow=True)     # sampled from before the next step
         samplers = [r for r, s in zip(plan.requests, plan.samples) if s]
         tokens = self.sampler.sample(logits, [r.temperature for r in samplers],
@@ -264,9 +282,54 @@ class Scheduler:
                 self._finish(r)
         return True
 
+    # -- decode steps with the host one step ahead ---------------------------------------------------
+    def _pipelinable(self, plan: StepPlan) -> bool:
+        """A step of single tokens that all sample, whose finishing does not depend on the tokens
+        (no stop tokens) and whose logits nobody keeps: it can be launched before the tokens of
+        the step before it have reached the host, which then are fed back on the device."""
+        if not self.async_decode or not self.runner.can_decode_async(len(plan.requests)):
+            return False
+        if any(n != 1 or not s or r.keep_logits for r, n, s in zip(plan.requests, plan.counts, plan.samples)):
+            return False
+        if self._inflight is not None:
+            before = self._inflight[1]
+            for r in plan.requests:
+                if r.generated and r.generated[-1] is None and r not in before:
+                    return False
+        return True
+
+    def _launch_decode(self, plan: StepPlan) -> None:
+        from ..sampling.sampler import _signed, row_key
+        reqs = plan.requests
+        tokens = [(r.generated[-1] if r.generated else r.prompt[-1]) for r in reqs]
+        keys = [_signed(row_key(self.sampler.seed, r.req_id, len(r.generated))) for r in reqs]
+        handle = self.runner.decode_launch([r.req_id for r in reqs], tokens, [r.temperature for r in reqs], keys)
+        previous, self._inflight = self._inflight, (handle, list(reqs), [len(r.generated) for r in reqs])
+        self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in reqs], counts=[1] * len(reqs),
+                                  sampled=[r.req_id for r in reqs]))
+        self.steps += 1
+        for r in reqs:
+            r.fed += 1
+            r.generated.append(None)          # filled in when the step's tokens are read back
+            if r.done():
+                self._finish(r)               # its pages may go to a later launch, which runs after this one
+        if previous is not None:
+            self._read_back(previous)
+
+    def _read_back(self, flight) -> None:
+        handle, reqs, places = flight
+        for r, i, tok in zip(reqs, places, handle.tokens()):
+            r.generated[i] = int(tok)
+
+    def _resolve(self) -> None:
+        if self._inflight is not None:
+            self._read_back(self._inflight)
+            self._inflight = None
+
     def run(self, requests: Sequence[GenerationRequest]) -> List[GenerationRequest]:
         """Generate for all requests; returns them in the order given."""
         self.add(requests)
         while self.step():
             pass
+        self._resolve()
         return list(requests)

@@ -112,7 +112,10 @@ class Model:
     # -- running -------------------------------------------------------------------------------
     def forward(self, ctx, caches: List[LayerCache]) -> torch.Tensor:
         """Run the tokens of one step; return fp32 logits [R, V] at ctx.logit_rows."""
-        x = self.embedding.forward(ctx.token_ids)
+        if getattr(ctx, "src_row", None) is not None:
+            x = self.embedding.forward(ctx.token_ids, ctx.src_row, ctx.prev_tokens)
+        else:
+            x = self.embedding.forward(ctx.token_ids)
         pending = None
         for e in self.spec.run_order:
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)

@@ -70,18 +70,23 @@ def _i32(t: torch.Tensor, n: int, name: str) -> None:
 
 # ---------------------------------------------------------------------------------------------
 
-def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = table[tokens[t]] as fp32.  Token ids must have been checked against the table
-    on the host (the batch builder does)."""
-    _dev(table, tokens, out)
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor,
+          src_row: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = table[tokens[t]] as fp32.  Where src_row[t] >= 0 the id is prev[src_row[t]] instead:
+    a token sampled on the device by an earlier step.  Host-given ids have been checked against
+    the table by the batch builder; the kernel clamps as a last resort."""
+    _dev(table, tokens, out, src_row, prev)
     T = tokens.numel()
     _check(table.dim() == 2, "embedding table must be [V, d]")
-    d = table.shape[1]
+    V, d = table.shape
     _i32(tokens, T, "tokens")
     _check(out.dtype == torch.float32 and out.shape == (T, d), "embed output must be fp32 [T, d]")
+    if src_row is not None:
+        _i32(src_row, T, "src_row")
+        _check(prev is not None and prev.dtype == torch.int32, "prev must be int32")
     lib = load_library("elementwise")
-    _ret(lib.sa_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out), c_int(T), c_int(d),
-                      _stream()), "embed")
+    _ret(lib.sa_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(src_row), _ptr(prev), _ptr(out),
+                      c_int(T), c_int(d), c_int(V), _stream()), "embed")
     return out
 
 
@@ -273,7 +278,7 @@ def split_k_parts(M: int, N: int, K: int) -> int:
         return 1
     tiles = -(-N // 16)
     parts = 1
-    while parts < 8 and tiles * parts < 1024 and K // (parts * 2) >= 512:
+    while parts < 4 and tiles * parts < 512 and K // (parts * 2) >= 512:
         parts *= 2
     return parts
 
@@ -301,6 +306,39 @@ def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> 
     _ret(lib.sa_gemm_bf16_skinny_swiglu(_ptr(a), _ptr(w_gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
                                         _stream()), "swiglu_bf16")
     return out
+
+
+def qkv_rope_available(a: torch.Tensor, w_qkv: torch.Tensor, k_pages: torch.Tensor, head_dim: int,
+                       rot_dim: int, adjacent_pairs: bool) -> bool:
+    """Whether projection, rotation and cache write can run as one kernel: bf16, few rows, all
+    dims of a head rotated in (j, j + D/2) pairs, head size a multiple of 32."""
+    return (a.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
+            and a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0 and head_dim % 32 == 0
+            and rot_dim == head_dim and not adjacent_pairs and _aligned16(a, w_qkv))
+
+
+def qkv_rope_bf16(a: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
+                  inv_freq: torch.Tensor, slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                  num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+    """q, k, v = a @ w_qkv^T (w_qkv = [Wq; Wk; Wv]); q and k rotated by position; q to q_out
+    [M, Hq D], rotated k and v into the cache pages at each token's slot.  One kernel."""
+    _dev(a, w_qkv, q_out, positions, inv_freq, slots, k_pages, v_pages)
+    M, K = a.shape
+    Hq, Hk, D = num_heads, num_kv_heads, head_dim
+    _check(qkv_rope_available(a, w_qkv, k_pages, D, D, False), "qkv_rope_bf16 does not take these operands")
+    _check(w_qkv.shape == ((Hq + 2 * Hk) * D, K), f"w_qkv must be [{(Hq + 2 * Hk) * D}, {K}]")
+    _check(q_out.shape == (M, Hq * D) and q_out.dtype == torch.bfloat16, "q_out must be bf16 [M, Hq D]")
+    _i32(positions, M, "positions")
+    _i32(slots, M, "slots")
+    _check(inv_freq.dtype == torch.float32 and inv_freq.numel() == D // 2, f"inv_freq must be fp32 [{D // 2}]")
+    P = k_pages.shape[0]
+    _check(k_pages.shape == (P, Hk, page_size, D) and v_pages.shape == (P, Hk, D, page_size)
+           and v_pages.dtype == torch.bfloat16, "cache pages must be bf16 [P, Hk, page, D] and [P, Hk, D, page]")
+    lib = load_library("gemm_mfma")
+    _ret(lib.sa_gemm_bf16_qkv_rope(_ptr(a), _ptr(w_qkv), _ptr(q_out), _ptr(positions), _ptr(inv_freq), _ptr(slots),
+                                   _ptr(k_pages), _ptr(v_pages), c_int(M), c_int(K), c_int(Hq), c_int(Hk),
+                                   c_int(D), c_int(page_size), _stream()), "qkv_rope_bf16")
+    return q_out
 
 
 MFMA_ATTENTION_HEAD_DIMS = tuple(range(16, 129, 16))

@@ -91,6 +91,19 @@ class RotaryPosition(Part):
         self.rt = rt
         self.inv_freq = rope_inverse_frequencies(self.rot_dim, self.theta, self.scaling).to(rt.device)
 
+    def project_rotate_store(self, h: torch.Tensor, w_qkv: torch.Tensor, positions: torch.Tensor,
+                             slots: torch.Tensor, cache: LayerCache, num_heads: int,
+                             num_kv_heads: int) -> Optional[torch.Tensor]:
+        """The q/k/v product, the rotation and the cache write as one kernel, where the kernel
+        takes the sizes: returns rotated q [T, Hq D], or None (then the caller does the steps
+        one by one)."""
+        if not ops.qkv_rope_available(h, w_qkv, cache.k_pages, self.head_dim, self.rot_dim,
+                                      self.pairing == "adjacent"):
+            return None
+        q = self.rt.empty((h.shape[0], num_heads * self.head_dim))
+        return ops.qkv_rope_bf16(h, w_qkv, q, positions, self.inv_freq, slots, cache.k_pages, cache.v_pages,
+                                 num_heads, num_kv_heads, self.head_dim, cache.page_size)
+
     def rotate_and_store(self, qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
                          cache: Optional[LayerCache], num_heads: int, num_kv_heads: int) -> None:
         ops.rope_kv_write(qkv, positions, self.inv_freq, slots,
@@ -142,7 +155,13 @@ class GQAAttention(Part):
     def forward(self, h: torch.Tensor, ctx, cache: LayerCache, writes_cache: bool = True) -> torch.Tensor:
         T = h.shape[0]
         grp = ctx.groups[cache.group]
-        if writes_cache:
+        fused = getattr(self.position, "project_rotate_store", None)
+        qkv = None
+        if writes_cache and fused is not None:
+            qkv = fused(h, self.wqkv, ctx.positions, grp.slots, cache, self.num_heads, self.num_kv_heads)
+        if qkv is not None:
+            pass                                # q alone, rotated; k and v are in the cache
+        elif writes_cache:
             qkv = linear(h, self.wqkv)
             self.position.rotate_and_store(qkv, ctx.positions, grp.slots, cache, self.num_heads,
                                            self.num_kv_heads)
@@ -208,9 +227,11 @@ class TokenEmbedding(Part):
         self.rt = rt
         self.weight = tensors["weight"]
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, token_ids: torch.Tensor, src_row: Optional[torch.Tensor] = None,
+                prev: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """`src_row` / `prev`: rows whose token was sampled on the device by an earlier step."""
         x = self.rt.empty((token_ids.numel(), self.hidden_size), torch.float32)
-        return ops.embed(self.weight, token_ids, x)
+        return ops.embed(self.weight, token_ids, x, src_row, prev)
 
 
 class LinearHead(Part):

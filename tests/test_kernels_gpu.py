@@ -431,3 +431,37 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
     torch.testing.assert_close(y.double(), ref, atol=2e-2, rtol=1e-2)
     assert ops.split_k_parts(8, 2048, 2048) > 1 and ops.split_k_parts(8, 16384, 2048) == 1
     assert ops.split_k_parts(64, 2048, 2048) == 1
+
+
+@pytest.mark.parametrize("M,Hq,Hk,D,ps,d", [(1, 4, 2, 32, 8, 64), (8, 32, 8, 64, 16, 2048), (13, 3, 1, 96, 4, 72),
+                                             (40, 6, 2, 128, 16, 200), (64, 2, 2, 64, 32, 96)])
+def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
+    from serve_amd import ops
+    P = 7
+    h = rnd((M, d), torch.bfloat16, 1)
+    w = rnd(((Hq + 2 * Hk) * D, d), torch.bfloat16, 2, 0.1)
+    pos = torch.randint(0, 3000, (M,), generator=torch.Generator().manual_seed(3)).to(torch.int32).to(DEV)
+    inv_freq = (1.0 / (500000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+    slots = torch.randperm(P * ps, generator=torch.Generator().manual_seed(4))[:M].to(torch.int32).to(DEV)
+    slots[0] = -1                                           # this token stores nothing
+    k1 = torch.zeros((P, Hk, ps, D), dtype=torch.bfloat16, device=DEV)
+    v1 = torch.zeros((P, Hk, D, ps), dtype=torch.bfloat16, device=DEV)
+    k2, v2 = k1.clone(), v1.clone()
+    assert ops.qkv_rope_available(h, w, k1, D, D, False)
+    q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=DEV)
+    ops.qkv_rope_bf16(h, w, q, pos, inv_freq, slots, k1, v1, Hq, Hk, D, ps)
+    # the same in three steps: product (fp32 out), rotation and write in fp32, rounding at the end
+    qkv = torch.empty((M, (Hq + 2 * Hk) * D), dtype=torch.float32, device=DEV)
+    ops.gemm_bf16_skinny(h, w, qkv)
+    x = qkv.double().view(M, Hq + 2 * Hk, D)
+    q_want = rope_ref(x[:, :Hq], pos, inv_freq, D, False).reshape(M, Hq * D)
+    k_want = rope_ref(x[:, Hq:Hq + Hk], pos, inv_freq, D, False)
+    torch.testing.assert_close(q.double(), q_want, atol=2e-2, rtol=1e-2)
+    ok = slots >= 0
+    page, off = (slots[ok] // ps).long(), (slots[ok] % ps).long()
+    torch.testing.assert_close(k1.double()[page, :, off, :], k_want[ok], atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(v1.double()[page, :, :, off], x[:, Hq + Hk:][ok], atol=2e-2, rtol=1e-2)
+    mask = torch.ones((P, ps), dtype=torch.bool, device=DEV)
+    mask[page, off] = False
+    assert k1.permute(0, 2, 1, 3)[mask].abs().max().item() == 0 and v1.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
+    assert not ops.qkv_rope_available(h, w, k1, 48, 48, False) and not ops.qkv_rope_available(h, w, k1, D, D, True)

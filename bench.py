@@ -118,6 +118,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=16, help="fewer than 16 only to save time; both are reported")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch-1/64 points")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiling); prints its own short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -137,6 +139,12 @@ def main() -> int:
     engine = Engine.from_config(cfg, seed=0, cfg=ecfg)
     print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
 
+    if args.prefill_only:
+        T = 2048
+        pt = prefill_run(engine, T, repeats=5, seed=7)
+        print(json.dumps({"prefill": {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                                      "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}}), flush=True)
+        return 0
     steps, warmup = args.steps, args.warmup
     prompt_len = args.context - (warmup + steps + 3)
     if prompt_len < 1:

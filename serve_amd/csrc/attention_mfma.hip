@@ -56,24 +56,19 @@ __device__ __forceinline__ uint32_t pack2bf(float a, float b) {
 // NT: column tiles (16 query rows each) per wave.  POW2: the page size is a power of two of at
 // least 8 (key -> page by shift, 16-byte value runs); otherwise any multiple of 4 (division,
 // 8-byte value runs).
+// One tile of one (segment, KV head, split): everything a wave does.
 template <int NT, bool POW2>
-__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
+__device__ __forceinline__ void attention_tile(
+    const int tile, const int seg, const int hk, const int sp, const int q_begin, const int q_len,
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
-    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
-    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ ctx_len, int Hq, int Hk,
+    int page_size, int page_shift, float scale_log2e, int window, int num_splits,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
   const int c = lane & 15;
-  const int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int hk = blockIdx.y;
-  const int seg = blockIdx.z / num_splits;
-  const int sp = blockIdx.z - seg * num_splits;
   const int G = Hq / Hk;
-
-  const int q_begin = cu_q[seg];
-  const int q_len = cu_q[seg + 1] - q_begin;
   const int rows_total = q_len * G;
   const int r0 = tile * (16 * NT);
   if (r0 >= rows_total) return;
@@ -238,7 +233,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       }
     }
 
-    // ---- online softmax over this lane's 8 keys per column, shared across the 4 lane groups
+    // ---- online softmax over this lane's 8 keys per column, shared across the 4 lane groups.
+    // The scale is positive, so the maximum is taken on the raw scores and the scale is applied
+    // inside the exponent: p = 2^(s * scale - m).
     Frag pf[NT];
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
@@ -248,7 +245,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float x = s[t][n][r] * scale_log2e;
+          float x = s[t][n][r];
           if (!full) {
             const int key = key0 + 8 * g + 4 * t + r;
             const bool vis = key <= qpos[n] && (window <= 0 || key > qpos[n] - window);
@@ -259,7 +256,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[n], mx);
+      const float m_new = fmaxf(m[n], mx * scale_log2e);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m[n] - m_safe);
       m[n] = m_new;
@@ -268,12 +265,15 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          v[t][r] = __builtin_amdgcn_exp2f(v[t][r] - m_safe);
+          v[t][r] = __builtin_amdgcn_exp2f(fmaf(v[t][r], scale_log2e, -m_safe));
           ps += v[t][r];
         }
       l[n] = l[n] * alpha + ps;
+      // the running maximum rarely moves after the first blocks: skip the rescaling then
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) acc[dt][n] *= alpha;
+        for (int dt = 0; dt < DT; ++dt) acc[dt][n] *= alpha;
+      }
       pf[n].u = make_uint4(pack2bf(v[0][0], v[0][1]), pack2bf(v[0][2], v[0][3]),
                            pack2bf(v[1][0], v[1][1]), pack2bf(v[1][2], v[1][3]));
     }
@@ -336,6 +336,40 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
 }
 
+// A wave takes tile w of its (segment, KV head).  With PAIR it takes tile ntiles-1-w as well: under
+// the causal mask tile t reads keys up to about t's end, so the two together are always one full
+// context long and all waves of a prompt finish at about the same time.
+template <int NT, bool POW2, bool PAIR>
+__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
+    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  const int w = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int hk = blockIdx.y;
+  const int seg = blockIdx.z / num_splits;
+  const int sp = blockIdx.z - seg * num_splits;
+  const int q_begin = cu_q[seg];
+  const int q_len = cu_q[seg + 1] - q_begin;
+  if (!PAIR) {
+    attention_tile<NT, POW2>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+                             max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
+                             part_o, part_ml);
+    return;
+  }
+  const int ntiles = (q_len * (Hq / Hk) + 16 * NT - 1) / (16 * NT);
+  if (w >= (ntiles + 1) / 2) return;                                  // the second half is done by pairing
+  attention_tile<NT, POW2>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+                           max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
+                           part_o, part_ml);
+  const int other = ntiles - 1 - w;
+  if (other > w)
+    attention_tile<NT, POW2>(other, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+                             max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
+                             part_o, part_ml);
+}
+
 // out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s; at most 64 splits.
 // One wave per (token, head): the lanes first share the work over the splits (weights), then over
 // the head dims (weighted sum, with independent loads that can all be in flight).
@@ -395,23 +429,28 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   const bool small = (long long)max_q_len * G <= 16;
   const int rows_per_tile = small ? 16 : 16 * NT_PREFILL;
   const int tiles = (int)(((long long)max_q_len * G + rows_per_tile - 1) / rows_per_tile);
-  dim3 grid((tiles + 3) / 4, Hk, B * num_splits), block(256);
+  // prompt portions: a wave takes tiles w and tiles-1-w, so half as many waves are launched
+  const bool pair = !small && num_splits == 1;
+  const int waves = pair ? (tiles + 1) / 2 : tiles;
+  dim3 grid((waves + 3) / 4, Hk, B * num_splits), block(256);
   const float scale_log2e = scale * 1.4426950408889634f;
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
   }
-#define GO(NT, POW2)                                                                                  \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT, POW2>), grid, block, 0, stream, (const bf16_t*)q, \
-                     q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
-                     block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, page_shift,            \
-                     scale_log2e, window, num_splits, part_o, part_ml)
+#define GO(NT, POW2, PAIR)                                                                             \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT, POW2, PAIR>), grid, block, 0, stream,            \
+                     (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages,                 \
+                     (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
+                     page_shift, scale_log2e, window, num_splits, part_o, part_ml)
   const bool pow2 = page_shift >= 3;
-  if (small && pow2) GO(1, true);
-  else if (small) GO(1, false);
-  else if (pow2) GO(NT_PREFILL, true);
-  else GO(NT_PREFILL, false);
+  if (small && pow2) GO(1, true, false);
+  else if (small) GO(1, false, false);
+  else if (pair && pow2) GO(NT_PREFILL, true, true);
+  else if (pair) GO(NT_PREFILL, false, true);
+  else if (pow2) GO(NT_PREFILL, true, false);
+  else GO(NT_PREFILL, false, false);
 #undef GO
   SA_LAUNCH_CHECK();
   if (num_splits > 1) {

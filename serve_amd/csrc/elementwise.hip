@@ -257,9 +257,38 @@ __global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ a, i
   }
 }
 
+// the same, eight bf16 values per thread in 16-byte vectors (I % 8 == 0)
+__global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ a,
+                                                               int T, int I) {
+  const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i >= I) return;
+  for (int t = blockIdx.y; t < T; t += gridDim.y) {
+    const uint4 gv = *reinterpret_cast<const uint4*>(gu + (size_t)t * 2 * I + i);
+    const uint4 uv = *reinterpret_cast<const uint4*>(gu + (size_t)t * 2 * I + I + i);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w};
+    const uint32_t uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float g0 = bf16_bits_to_float(gw[k] & 0xffffu), g1 = bf16_bits_to_float(gw[k] >> 16);
+      const float u0 = bf16_bits_to_float(uw[k] & 0xffffu), u1 = bf16_bits_to_float(uw[k] >> 16);
+      const float o0 = (g0 / (1.f + expf(-g0))) * u0;
+      const float o1 = (g1 / (1.f + expf(-g1))) * u1;
+      ow[k] = (uint32_t)float_to_bf16_bits(o0) | ((uint32_t)float_to_bf16_bits(o1) << 16);
+    }
+    *reinterpret_cast<uint4*>(a + (size_t)t * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 extern "C" int sa_silu_mul(const void* gu, void* a, int act_dtype, int T, int I, hipStream_t stream) {
   if (T <= 0) return 0;
   if (I <= 0) return SA_ERR_ARG;
+  if (act_dtype == SA_BF16 && (I & 7) == 0) {
+    dim3 grid((I / 8 + 255) / 256, T < 32768 ? T : 32768), block(256);
+    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)a, T, I);
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((I + 255) / 256, T < 32768 ? T : 32768), block(256);
   if (act_dtype == SA_F32)
     hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)a, T, I);

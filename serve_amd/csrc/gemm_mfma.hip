@@ -1,8 +1,9 @@
 // bf16 matrix products on the matrix cores for few rows of activations (decode steps and short
 // prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
+// Two kernels: gemm_skinny_kernel for up to 16 rows, gemm_mid_kernel for 17 to 64 (per pass).
 //
-// The work is bound by reading W.  A wave owns RT tiles of 16 rows of W and walks a slice of K in
-// steps of 32; the KS waves of a workgroup split K between them and add their partial sums
+// The work is bound by reading W.  In the first, a wave owns RT tiles of 16 rows of W and walks a
+// slice of K in steps of 32; the KS waves of a workgroup split K between them and add their partial sums
 // through LDS, so no atomics and a fixed summation order.  The MFMA computes the transposed
 // tile: operand "A" of v_mfma_f32_16x16x32_bf16 is a 16x32 tile of W (lane l: row l%16, k-slots
 // 8*(l/16)..+7), operand "B" is 32x16 of activations (lane l: activation row l%16, same k-slots),
@@ -17,9 +18,11 @@
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 union Frag {
   uint4 u;
+  u32x4_t r;
   bf16x8_t v;
 };
 
@@ -43,121 +46,13 @@ struct QkvRopeArgs {
   int Hq, Hk, D, page_size;
 };
 
-template <int RT, int MT, int KS, int KU, typename TC, int EPI, bool STREAM = false>
-__global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
-                                                             const bf16_t* __restrict__ W,
-                                                             TC* __restrict__ C, int M, int N, int K,
-                                                             int up_offset, QkvRopeArgs qa) {
+// What is done with a wave's finished sums acc[rt][mt] (lane l: activation row m0 + 16 mt + l%16,
+// outputs 4*(l/16) .. +3 of row tile rt); the row tiles start at n0 as the kernels below lay them out.
+template <int RT, int MT, typename TC, int EPI>
+__device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __restrict__ C, int M, int N, int m0,
+                                            int n0, int head, int t16, const QkvRopeArgs& qa, int g, int c) {
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
   constexpr bool QKV = EPI == EPI_QKV_ROPE;
-  static_assert(KS * RT * MT <= 64, "partial sums must fit into 64 KB of LDS");
-  static_assert(EPI == EPI_PLAIN || RT == 2, "the pairing epilogues work on two row tiles");
-  __shared__ float red[KS][RT * MT * 4][64];
-
-  const int wave = threadIdx.x >> 6;
-  const int lane = threadIdx.x & 63;
-  const int g = lane >> 4;
-  const int c = lane & 15;
-  // first row of this workgroup's (first) tile; QKV: tile t16 of head `head`, second tile D/2 below
-  const int tph = QKV ? (qa.D >> 5) : 1;
-  const int head = QKV ? blockIdx.x / tph : 0;
-  const int t16 = QKV ? blockIdx.x - head * tph : 0;
-  const int n0 = QKV ? head * qa.D + t16 * 16 : blockIdx.x * (SWIGLU ? 16 : RT * 16);
-  const int m0 = blockIdx.y * (MT * 16);
-
-  const int nchunks = (K + 31) >> 5;
-  const int per_wg = (nchunks + gridDim.z - 1) / gridDim.z;
-  const int wg_begin = blockIdx.z * per_wg;
-  const int wg_end = min(nchunks, wg_begin + per_wg);
-  const int per = (per_wg + KS - 1) / KS;
-  const int ch_begin = wg_begin + wave * per;
-  const int ch_end = min(wg_end, ch_begin + per);
-  C += (size_t)blockIdx.z * M * N;
-
-  const bf16_t* wrow[RT];
-  bool wok[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    int n;
-    if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
-    else if (QKV) n = n0 + rt * (qa.D >> 1) + c;
-    else n = n0 + rt * 16 + c;
-    wok[rt] = SWIGLU ? (n0 + c < N) : (n < N);
-    wrow[rt] = W + (size_t)(wok[rt] ? n : 0) * K;
-  }
-  const bf16_t* arow[MT];
-  bool aok[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = m0 + mt * 16 + c;
-    aok[mt] = m < M;
-    arow[mt] = A + (size_t)(aok[mt] ? m : 0) * K;
-  }
-
-  floatx4_t acc[RT][MT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  for (int ch = ch_begin; ch < ch_end; ch += KU) {
-    Frag wf[RT][KU], af[MT][KU];
-#pragma unroll
-    for (int u = 0; u < KU; ++u) {
-      const int k = (ch + u) * 32 + g * 8;
-      const bool kin = (ch + u) < ch_end && k < K;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        wf[rt][u].u = zero;
-        if (kin && wok[rt]) {
-          const uint4* src = reinterpret_cast<const uint4*>(wrow[rt] + k);
-          if (STREAM) {
-            typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-            const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
-            wf[rt][u].u = make_uint4(t.x, t.y, t.z, t.w);
-          } else {
-            wf[rt][u].u = *src;
-          }
-        }
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        af[mt][u].u = zero;
-        if (kin && aok[mt]) af[mt][u].u = *reinterpret_cast<const uint4*>(arow[mt] + k);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < KU; ++u)
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][u].v, af[mt][u].v, acc[rt][mt], 0, 0, 0);
-  }
-
-  // add the KS partial sums in a fixed order: every wave stores, wave 0 sums and writes
-  if (KS > 1) {
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) red[wave][(rt * MT + mt) * 4 + r][lane] = acc[rt][mt][r];
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float s = acc[rt][mt][r];
-          for (int w = 1; w < KS; ++w) s += red[w][(rt * MT + mt) * 4 + r][lane];
-          acc[rt][mt][r] = s;
-        }
-  }
-
   const int ldc = N;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -234,6 +129,347 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   }
 }
 
+template <int RT, int MT, int KS, int KU, typename TC, int EPI, bool STREAM = false>
+__global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
+                                                             const bf16_t* __restrict__ W,
+                                                             TC* __restrict__ C, int M, int N, int K,
+                                                             int up_offset, QkvRopeArgs qa) {
+  constexpr bool SWIGLU = EPI == EPI_SWIGLU;
+  constexpr bool QKV = EPI == EPI_QKV_ROPE;
+  static_assert(KS * RT * MT <= 64, "partial sums must fit into 64 KB of LDS");
+  static_assert(EPI == EPI_PLAIN || RT == 2, "the pairing epilogues work on two row tiles");
+  __shared__ float red[KS][RT * MT * 4][64];
+
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  // first row of this workgroup's (first) tile; QKV: tile t16 of head `head`, second tile D/2 below
+  const int tph = QKV ? (qa.D >> 5) : 1;
+  const int head = QKV ? blockIdx.x / tph : 0;
+  const int t16 = QKV ? blockIdx.x - head * tph : 0;
+  const int n0 = QKV ? head * qa.D + t16 * 16 : blockIdx.x * (SWIGLU ? 16 : RT * 16);
+  const int m0 = blockIdx.y * (MT * 16);
+
+  const int nchunks = (K + 31) >> 5;
+  const int per_wg = (nchunks + gridDim.z - 1) / gridDim.z;
+  const int wg_begin = blockIdx.z * per_wg;
+  const int wg_end = min(nchunks, wg_begin + per_wg);
+  const int per = (per_wg + KS - 1) / KS;
+  const int ch_begin = wg_begin + wave * per;
+  const int ch_end = min(wg_end, ch_begin + per);
+  C += (size_t)blockIdx.z * M * N;
+
+  const bf16_t* wrow[RT];
+  bool wok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    int n;
+    if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
+    else if (QKV) n = n0 + rt * (qa.D >> 1) + c;
+    else n = n0 + rt * 16 + c;
+    wok[rt] = SWIGLU ? (n0 + c < N) : (n < N);
+    wrow[rt] = W + (size_t)(wok[rt] ? n : 0) * K;
+  }
+  const bf16_t* arow[MT];
+  bool aok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + mt * 16 + c;
+    aok[mt] = m < M;
+    arow[mt] = A + (size_t)(aok[mt] ? m : 0) * K;
+  }
+
+  floatx4_t acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int ch = ch_begin; ch < ch_end; ch += KU) {
+    Frag wf[RT][KU], af[MT][KU];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int k = (ch + u) * 32 + g * 8;
+      const bool kin = (ch + u) < ch_end && k < K;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        wf[rt][u].u = zero;
+        if (kin && wok[rt]) {
+          const uint4* src = reinterpret_cast<const uint4*>(wrow[rt] + k);
+          if (STREAM) {
+            const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
+            wf[rt][u].u = make_uint4(t.x, t.y, t.z, t.w);
+          } else {
+            wf[rt][u].u = *src;
+          }
+        }
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        af[mt][u].u = zero;
+        if (kin && aok[mt]) af[mt][u].u = *reinterpret_cast<const uint4*>(arow[mt] + k);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < KU; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][u].v, af[mt][u].v, acc[rt][mt], 0, 0, 0);
+  }
+
+  // add the KS partial sums in a fixed order: every wave stores, wave 0 sums and writes
+  if (KS > 1) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][(rt * MT + mt) * 4 + r][lane] = acc[rt][mt][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float s = acc[rt][mt][r];
+          for (int w = 1; w < KS; ++w) s += red[w][(rt * MT + mt) * 4 + r][lane];
+          acc[rt][mt][r] = s;
+        }
+  }
+
+  store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, g, c);
+}
+
+// The same products for 17..64 rows of activations (decode at larger batches, short prompt
+// portions).  With that many rows a workgroup reads about as many bytes of activations as of
+// weights, so the activations are staged through LDS and shared.  A workgroup has NR x KH waves:
+// NR groups of weight rows times KH slices of each 256-wide stage of K; the NR waves of a slice read
+// the same activation fragments, and the KH slices add their sums through LDS at the end, in order.
+// Weight fragments go from global memory straight into registers, two stages ahead of the products;
+// activations are loaded one stage ahead into registers and written to the LDS buffer of their
+// stage (two buffers in turn: one barrier per stage).  A row of a stage holds 32 segments of
+// 16 bytes; segment s of row r is stored at slot s ^ (r % 16), which makes both the stores (16 lanes
+// along a row) and the fragment reads (16 lanes along a column of segments) free of bank conflicts.
+template <int RT, int MT, int NR, int KH, typename TC, int EPI>
+__global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __restrict__ A,
+                                                                const bf16_t* __restrict__ W,
+                                                                TC* __restrict__ C, int M, int N, int K,
+                                                                int up_offset, QkvRopeArgs qa) {
+  constexpr bool SWIGLU = EPI == EPI_SWIGLU;
+  constexpr bool QKV = EPI == EPI_QKV_ROPE;
+  static_assert(EPI == EPI_PLAIN || RT == 2, "the pairing epilogues work on two row tiles");
+  static_assert(KH == 2 || KH == 4 || KH == 8, "a stage is 8 steps of 32");
+  constexpr int THREADS = 64 * NR * KH;
+  constexpr int ROWS = MT * 16;            // activation rows of a workgroup
+  constexpr int NA = ROWS * 32 / THREADS;  // 16-byte activation segments per thread and stage
+  constexpr int KU = 8 / KH;               // steps of 32 per wave and stage
+  static_assert(ROWS * 32 % THREADS == 0, "the activation tile is spread evenly over the threads");
+  __shared__ u32x4_t lds[2][ROWS][32];     // [buffer][row][segment slot]
+  static_assert(sizeof(lds) >= (size_t)(KH - 1) * NR * RT * MT * 4 * 64 * sizeof(float),
+                "the sums of the other K slices reuse it");
+
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int rg = wave % NR;                // row group
+  const int kh = wave / NR;                // K slice
+  const int tile = blockIdx.x * NR + rg;
+  const int tph = QKV ? (qa.D >> 5) : 1;
+  const int head = QKV ? tile / tph : 0;
+  const int t16 = QKV ? tile - head * tph : 0;
+  const int n0 = QKV ? head * qa.D + t16 * 16 : tile * (SWIGLU ? 16 : RT * 16);
+  const int m0 = blockIdx.y * ROWS;
+
+  // this workgroup's slice of K, in chunks of 32
+  const int nchunks = (K + 31) >> 5;
+  const int per_wg = (nchunks + gridDim.z - 1) / gridDim.z;
+  const int k_begin = blockIdx.z * per_wg * 32;
+  const int k_end = min(K, k_begin + per_wg * 32);
+  const int nstages = (k_end - k_begin + 255) >> 8;
+  // Workgroups walk their stages in rotated order.  All of them read the same few activation rows,
+  // whose stride is often a power of two: the same K offset of every row then lies in the same L2
+  // channel, and workgroups in step would queue there.  (The order depends on the weight rows
+  // only, so a row of activations gets the same sums whatever else is in the batch.)
+  const int rot = nstages > 0 ? (int)(blockIdx.x % (unsigned)nstages) : 0;
+  auto stage_k = [&](int s) __attribute__((always_inline)) {
+    int t = s + rot;
+    if (t >= nstages) t -= nstages;
+    return k_begin + t * 256;
+  };
+  C += (size_t)blockIdx.z * M * N;
+
+  const bf16_t* wrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    int n;
+    if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
+    else if (QKV) n = n0 + rt * (qa.D >> 1) + c;
+    else n = n0 + rt * 16 + c;
+    bool ok = SWIGLU ? (n0 + c < N) : (n < N);
+    if (QKV) ok = head < qa.Hq + 2 * qa.Hk;
+    wrow[rt] = W + (size_t)(ok ? n : 0) * K;
+  }
+  // the activation segments this thread moves: row idx / 32, 16-byte segment idx % 32 of the stage
+  const bf16_t* asrc[NA];
+  int aseg[NA];
+  u32x4_t* adst[NA];
+#pragma unroll
+  for (int j = 0; j < NA; ++j) {
+    const int idx = threadIdx.x + THREADS * j;
+    const int row = idx >> 5;
+    const int seg = idx & 31;
+    asrc[j] = A + (size_t)(m0 + row < M ? m0 + row : 0) * K;
+    aseg[j] = seg;
+    adst[j] = &lds[0][row][seg ^ (row & 15)];
+  }
+
+  floatx4_t acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+  // Loads carry no per-lane conditions (a branch around every load would serialize them): rows
+  // beyond M or N are read from row 0 and give sums that are never stored, and beyond the end of
+  // the slice of K the address is clamped and the activation operand is zeroed on its way into LDS,
+  // which zeroes the product whatever finite weight stands there.
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
+  u32x4_t areg[NA];
+  auto load_acts = [&](int s) __attribute__((always_inline)) {
+    const int k0 = stage_k(s);
+#pragma unroll
+    for (int j = 0; j < NA; ++j)
+      areg[j] = *reinterpret_cast<const u32x4_t*>(asrc[j] + min(k0 + aseg[j] * 8, K - 8));
+  };
+  auto load_weights = [&](int s, Frag (&wf)[RT][KU]) __attribute__((always_inline)) {
+    const int k0 = stage_k(s) + kh * (KU * 32) + g * 8;
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int k = min(k0 + u * 32, K - 8);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) wf[rt][u].r = *reinterpret_cast<const u32x4_t*>(wrow[rt] + k);
+    }
+  };
+  // one stage: publish its activations, start the loads of what comes next (activations one
+  // stage ahead, weights two), multiply
+  auto stage = [&](int s, Frag (&cur)[RT][KU], Frag (&pre)[RT][KU]) __attribute__((always_inline)) {
+    constexpr int BUF = ROWS * 32;                      // 16-byte slots per buffer
+    const int b = s & 1;
+    const int k0 = stage_k(s);
+    if (k0 + 256 > k_end) {          // the zeroing waits for the loads, so it is done here and not where they start
+#pragma unroll
+      for (int j = 0; j < NA; ++j) areg[j] = k0 + aseg[j] * 8 < k_end ? areg[j] : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < NA; ++j) adst[j][b * BUF] = areg[j];
+    __syncthreads();
+    // (unconditional, so that the number of loads in flight is known where their results are
+    // awaited; past the last stage they read it again and nobody uses them)
+    load_acts(min(s + 1, nstages - 1));
+    load_weights(min(s + 2, nstages - 1), pre);
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      Frag af[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) af[mt].r = lds[b][mt * 16 + c][(kh * (KU * 4) + u * 4 + g) ^ c];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[rt][u].v, af[mt].v, acc[rt][mt], 0, 0, 0);
+    }
+  };
+
+  Frag w0[RT][KU], w1[RT][KU], w2[RT][KU];
+  if (nstages > 0) {
+    load_acts(0);
+    load_weights(0, w0);
+    load_weights(min(1, nstages - 1), w1);
+  }
+  // three stages a turn so that the register sets take turns without copies; the turn has no
+  // branches inside, which keeps the compiler's count of loads in flight exact
+  int s = 0;
+  for (; s + 3 <= nstages; s += 3) {
+    stage(s, w0, w2);
+    stage(s + 1, w1, w0);
+    stage(s + 2, w2, w1);
+  }
+  if (s < nstages) {
+    stage(s, w0, w2);
+    if (s + 1 < nstages) stage(s + 1, w1, w0);
+  }
+
+  // add the slices of K in a fixed order: the waves of slices 1.. hand their sums over through LDS
+  float* red = reinterpret_cast<float*>(&lds[0][0][0]);
+  __syncthreads();
+  if (kh > 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          red[((((kh - 1) * NR + rg) * RT * MT + rt * MT + mt) * 4 + r) * 64 + lane] = acc[rt][mt][r];
+  }
+  __syncthreads();
+  if (kh > 0) return;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float sum = acc[rt][mt][r];
+#pragma unroll
+        for (int h = 1; h < KH; ++h) sum += red[((((h - 1) * NR + rg) * RT * MT + rt * MT + mt) * 4 + r) * 64 + lane];
+        acc[rt][mt][r] = sum;
+      }
+  if (QKV && head >= qa.Hq + 2 * qa.Hk) return;
+  store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, g, c);
+}
+
+template <int RT, int MT, int NR, int KH, typename TC, int EPI>
+static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
+                      const QkvRopeArgs& qa, hipStream_t stream) {
+  unsigned tiles;
+  if (EPI == EPI_SWIGLU) tiles = (N + 15) / 16;
+  else if (EPI == EPI_QKV_ROPE) tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 5);
+  else tiles = (N + RT * 16 - 1) / (RT * 16);
+  dim3 grid((tiles + NR - 1) / NR, (M + MT * 16 - 1) / (MT * 16), parts);
+  if (grid.y > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
+  hipLaunchKernelGGL((gemm_mid_kernel<RT, MT, NR, KH, TC, EPI>), grid, dim3(64 * NR * KH), 0, stream,
+                     (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, up_offset, qa);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename TC, int EPI>
+static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
+                    const QkvRopeArgs& qa, hipStream_t stream) {
+  const bool four = M > 32;
+#define GO(RT, MT, NR, KH) \
+  return launch_mid<RT, MT, NR, KH, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
+  if constexpr (EPI == EPI_PLAIN) {
+    if (N < 8192) {                  // few weight rows: 32 a workgroup, K cut four ways inside it
+      if (four) GO(1, 4, 2, 4);
+      GO(1, 2, 2, 4);
+    }
+    if (four) GO(2, 4, 4, 2);        // many: 128 a workgroup, which halves the activation traffic
+    GO(2, 2, 4, 2);
+  }
+  if (four) GO(2, 4, 2, 4);
+  GO(2, 2, 2, 4);
+#undef GO
+  return SA_ERR_ARG;
+}
+
 template <int RT, int MT, int KS, int KU, typename TC, int EPI>
 static int launch_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
                          int parts, const QkvRopeArgs& qa, hipStream_t stream) {
@@ -252,34 +488,17 @@ static int launch_skinny(const void* A, const void* W, void* C, int M, int N, in
 template <typename TC, int EPI>
 static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
                        int parts, const QkvRopeArgs& qa, hipStream_t stream) {
-  // rows of activations per workgroup: 16, 32 or 64 (larger M loops over grid.y)
-  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  // many weight rows: 2 row tiles per wave and few waves; few rows: more waves splitting K
+  // up to 16 rows of activations (more take the kernel above; still more would loop over grid.y).
+  // Many weight rows: 2 row tiles per wave and few waves; few rows: more waves splitting K.
   const bool wide = EPI == EPI_SWIGLU || N >= 8192;
 #define GO(RT, MT, KS, KU) \
   return launch_skinny<RT, MT, KS, KU, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
   // (the choices below are the best of a sweep over RT, KS and KU at the Llama-3.2-1B sizes)
-  if constexpr (EPI == EPI_QKV_ROPE) {
-    if (mt == 1) GO(2, 1, 8, 8);
-    if (mt == 2) GO(2, 2, 8, 4);
-    GO(2, 4, 4, 4);
-  }
-  if (wide) {
-    if (mt == 1) GO(2, 1, 2, 8);
-    if (mt == 2) GO(2, 2, 4, 4);
-    GO(2, 4, 4, 4);
-  }
+  if constexpr (EPI == EPI_QKV_ROPE) GO(2, 1, 8, 8);
+  if (wide) GO(2, 1, 2, 8);
   if constexpr (EPI == EPI_PLAIN) {
-    if (parts > 1) {
-      // K is already cut across workgroups: 2 waves each
-      if (mt == 1) GO(1, 1, 2, 8);
-      if (mt == 2) GO(1, 2, 4, 4);
-      GO(1, 4, 4, 4);
-    }
-    // 16 waves leave 128 registers a lane, enough only for one activation tile
-    if (mt == 1) GO(1, 1, 16, 4);
-    if (mt == 2) GO(1, 2, 8, 4);
-    GO(1, 4, 8, 4);
+    if (parts > 1) GO(1, 1, 2, 8);   // K is already cut across workgroups: 2 waves each
+    GO(1, 1, 16, 4);
   }
 #undef GO
   return SA_ERR_ARG;
@@ -292,6 +511,11 @@ extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || parts < 1) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
+  if (M > 16) {
+    if (c_dtype == SA_BF16 && parts == 1) return pick_mid<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
+    if (c_dtype == SA_F32) return pick_mid<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
+    return SA_ERR_UNSUPPORTED;
+  }
   if (c_dtype == SA_BF16 && parts == 1) return pick_skinny<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
   if (c_dtype == SA_F32) return pick_skinny<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
   return SA_ERR_UNSUPPORTED;
@@ -303,6 +527,7 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
   if (M <= 0 || I <= 0) return 0;
   if (K <= 0 || (K & 7)) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
+  if (M > 16) return pick_mid<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   return pick_skinny<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
 }
 
@@ -315,5 +540,6 @@ extern "C" int sa_gemm_bf16_qkv_rope(const void* A, const void* W, void* Q, cons
   if (M <= 0) return 0;
   if (K <= 0 || (K & 7) || Hq <= 0 || Hk <= 0 || D <= 0 || (D & 31) || page_size <= 0) return SA_ERR_ARG;
   const QkvRopeArgs qa = {positions, inv_freq, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size};
+  if (M > 16) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   return pick_skinny<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
 }

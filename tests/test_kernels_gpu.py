@@ -368,7 +368,7 @@ def test_gemm_bf16_skinny(c_dt, M, N, K):
         torch.testing.assert_close(out2.double(), want, atol=2e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 192, 64), (8, 8192, 2048), (20, 320, 192), (64, 1000, 96)])
+@pytest.mark.parametrize("M,I,K", [(1, 192, 64), (8, 8192, 2048), (20, 320, 192), (64, 1000, 96), (50, 8192, 2048)])
 def test_swiglu_bf16(M, I, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 6)
@@ -409,7 +409,8 @@ def test_kernels_refuse_what_they_do_not_take():
                                    torch.zeros(1, dtype=torch.int32, device=DEV), 1, 1, 1.0, None)
 
 
-@pytest.mark.parametrize("M,N,K,parts", [(1, 2048, 2048, 4), (8, 2048, 8192, 2), (16, 96, 256, 8), (5, 77, 520, 3)])
+@pytest.mark.parametrize("M,N,K,parts", [(1, 2048, 2048, 4), (8, 2048, 8192, 2), (16, 96, 256, 8), (5, 77, 520, 3),
+                                         (40, 130, 1000, 3), (64, 2048, 2048, 4), (17, 48, 8192, 8)])
 def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 4)
@@ -430,7 +431,7 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
     ref = xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + 1e-5) * g.double()
     torch.testing.assert_close(y.double(), ref, atol=2e-2, rtol=1e-2)
     assert ops.split_k_parts(8, 2048, 2048) > 1 and ops.split_k_parts(8, 16384, 2048) == 1
-    assert ops.split_k_parts(64, 2048, 2048) == 1
+    assert ops.split_k_parts(64, 2048, 2048) > 1 and ops.split_k_parts(64, 128256, 2048) == 1
 
 
 @pytest.mark.parametrize("M,Hq,Hk,D,ps,d", [(1, 4, 2, 32, 8, 64), (8, 32, 8, 64, 16, 2048), (13, 3, 1, 96, 4, 72),

@@ -46,6 +46,21 @@ struct QkvRopeArgs {
   int Hq, Hk, D, page_size;
 };
 
+// sin and cos of an angle of up to about 2e5 rad (a position times a frequency of at most 1), to
+// about 1e-6: the library's sincosf spends over a thousand cycles on arguments this large.  The
+// multiple of 2 pi is taken off in three steps whose constants have few enough bits for the first
+// products to be exact (6.28125 = 201/32; 2029/2^20; the rest), the remainder goes to the
+// hardware's sine and cosine, which take their argument in turns.
+__device__ __forceinline__ void sincos_reduced(float x, float* sn, float* cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.28125f, x);
+  r = fmaf(-k, 1.93500518798828125e-3f, r);
+  r = fmaf(-k, 3.0199159776e-7f, r);
+  const float t = r * 0.15915494309189535f;
+  *sn = __builtin_amdgcn_sinf(t);
+  *cs = __builtin_amdgcn_cosf(t);
+}
+
 // What is done with a wave's finished sums acc[rt][mt] (lane l: activation row m0 + 16 mt + l%16,
 // outputs 4*(l/16) .. +3 of row tile rt); the row tiles start at n0 as the kernels below lay them out.
 template <int RT, int MT, typename TC, int EPI>
@@ -82,7 +97,7 @@ __device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __rest
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float sn, cs;
-          sincosf(pos * qa.inv_freq[dim0 + r], &sn, &cs);
+          sincos_reduced(pos * qa.inv_freq[dim0 + r], &sn, &cs);
           const float a = lo[r], b = hi[r];
           lo[r] = a * cs - b * sn;
           hi[r] = b * cs + a * sn;
@@ -463,6 +478,10 @@ static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, 
     }
     if (four) GO(2, 4, 4, 2);        // many: 128 a workgroup, which halves the activation traffic
     GO(2, 2, 4, 2);
+  }
+  if constexpr (EPI == EPI_QKV_ROPE) {  // few rows again: one pair of tiles a workgroup, K cut eight ways
+    if (four) GO(2, 4, 1, 8);
+    GO(2, 2, 1, 8);
   }
   if (four) GO(2, 4, 2, 4);
   GO(2, 2, 2, 4);

@@ -435,13 +435,14 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
 
 
 @pytest.mark.parametrize("M,Hq,Hk,D,ps,d", [(1, 4, 2, 32, 8, 64), (8, 32, 8, 64, 16, 2048), (13, 3, 1, 96, 4, 72),
-                                             (40, 6, 2, 128, 16, 200), (64, 2, 2, 64, 32, 96)])
+                                             (40, 6, 2, 128, 16, 200), (64, 2, 2, 64, 32, 96), (16, 5, 1, 64, 8, 520)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
     P = 7
     h = rnd((M, d), torch.bfloat16, 1)
     w = rnd(((Hq + 2 * Hk) * D, d), torch.bfloat16, 2, 0.1)
-    pos = torch.randint(0, 3000, (M,), generator=torch.Generator().manual_seed(3)).to(torch.int32).to(DEV)
+    # positions up to 131,071: the kernel takes the multiple of 2 pi off the angle itself
+    pos = torch.randint(0, 3000 if M < 40 else 131072, (M,), generator=torch.Generator().manual_seed(3)).to(torch.int32).to(DEV)
     inv_freq = (1.0 / (500000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
     slots = torch.randperm(P * ps, generator=torch.Generator().manual_seed(4))[:M].to(torch.int32).to(DEV)
     slots[0] = -1                                           # this token stores nothing

@@ -53,11 +53,28 @@ __device__ __forceinline__ uint32_t pack2bf(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
-// NT: column tiles (16 query rows each) per wave.  POW2: the page size is a power of two of at
-// least 8 (key -> page by shift, 16-byte value runs); otherwise any multiple of 4 (division,
-// 8-byte value runs).
+// maximum over the four lanes l, l^16, l^32, l^48 (the four lane groups of a column) with the row
+// swaps of gfx950 instead of two trips through LDS
+__device__ __forceinline__ float max_across_groups(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const uint32_t v = __float_as_uint(y);
+  const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+struct Masked { static constexpr bool value = true; };
+struct Unmasked { static constexpr bool value = false; };
+
+// NT: column tiles (16 query rows each) per wave.  PM: how keys map to pages:
+//   0  any page size that is a multiple of 4: division per key, 8-byte value runs;
+//   1  a power of two of at least 8: shift, 16-byte value runs; a block of 32 keys spans up to four
+//      pages and each lane picks its own;
+//   2  a power of two of at least 32: a block lies in one page, and every address is a scalar base
+//      plus a constant of the lane.
 // One tile of one (segment, KV head, split): everything a wave does.
-template <int NT, bool POW2>
+template <int NT, int PM>
 __device__ __forceinline__ void attention_tile(
     const int tile, const int seg, const int hk, const int sp, const int q_begin, const int q_len,
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -85,6 +102,10 @@ __device__ __forceinline__ void attention_tile(
   // the same for every lane: say so, or the integer division makes the whole loop control vector work
   const int b0 = __builtin_amdgcn_readfirstlane(kb_lo + sp * per);
   const int b1 = __builtin_amdgcn_readfirstlane(min(kb_hi + 1, b0 + per));
+  // blocks full_lo .. full_hi are visible as a whole to every row of the tile and need no mask:
+  // their last key is at most the first row's position, their first key inside the last row's window
+  const int full_hi = __builtin_amdgcn_readfirstlane((ctx_before + j_lo - 31) >> 5);
+  const int full_lo = window > 0 ? __builtin_amdgcn_readfirstlane(((ctx_before + j_hi - window) >> 5) + 1) : 0;
   const int* bt = block_table + (size_t)seg * max_pages;
 
   // this lane's query column in each column tile
@@ -119,7 +140,7 @@ __device__ __forceinline__ void attention_tile(
   }
 
   const size_t k_page_stride = (size_t)Hk * page_size * HD;   // elements per page (K and V alike)
-  constexpr bool wide_v = POW2;                                // 8 consecutive keys lie in one page
+  constexpr bool wide_v = PM >= 1;                             // 8 consecutive keys lie in one page
 
   // Which key sits in which row of the two 16-key tiles is free to choose.  Row i of tile t holds
   // key 8*(i/4) + 4*t + (i%4) of the block, so that after S^T = K Q^T lane group g holds the
@@ -131,40 +152,65 @@ __device__ __forceinline__ void attention_tile(
   // Page ids.  With a power-of-two page size a block of 32 keys spans at most four pages, the
   // same for every lane: they are fetched with scalar loads one block ahead (`pgn`), which keeps
   // them out of the vector-memory queue, so that waiting for them does not drain the K/V loads.
-  const int last_idx = POW2 ? ((ctx - 1) >> page_shift) : 0;
-  const int ppb_shift = POW2 ? page_shift : 0;
+  const int last_idx = PM >= 1 ? ((ctx - 1) >> page_shift) : 0;
   int pgn[4] = {0, 0, 0, 0};
-  auto prefetch_pages = [&](int kb) {
-    if (POW2) {
-      const int first = (kb << 5) >> ppb_shift;
+  auto prefetch_pages = [&](int kb) __attribute__((always_inline)) {
+    if (PM == 1) {
+      const int first = (kb << 5) >> page_shift;
+      int raw[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int idx = __builtin_amdgcn_readfirstlane(min(first + j, last_idx));
-        pgn[j] = __builtin_amdgcn_readfirstlane(max(bt[idx], 0));
-      }
+      for (int j = 0; j < 4; ++j) raw[j] = bt[__builtin_amdgcn_readfirstlane(min(first + j, last_idx))];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pgn[j] = __builtin_amdgcn_readfirstlane(max(raw[j], 0));
+    } else if (PM == 2) {
+      const int idx = __builtin_amdgcn_readfirstlane(min(kb >> (page_shift - 5), last_idx));
+      pgn[0] = __builtin_amdgcn_readfirstlane(max(bt[idx], 0));
     }
   };
-  auto pick = [&](const int (&pg)[4], int j) {          // two-level select, no branches
+  auto pick = [&](const int (&pg)[4], int j) __attribute__((always_inline)) {   // two-level select, no branches
     const int lo = (j & 1) ? pg[1] : pg[0];
     const int hi = (j & 1) ? pg[3] : pg[2];
     return (j & 2) ? hi : lo;
   };
   // key index -> (page, offset in the page) for page sizes that are no power of two
-  auto locate = [&](int key, int& page, int& off) {
+  auto locate = [&](int key, int& page, int& off) __attribute__((always_inline)) {
     const int idx = key / page_size;
     off = key - idx * page_size;
     page = max(bt[idx], 0);
   };
-  auto load_block = [&](int kb, Block& blk) {
+  // PM 2: where this lane's 16 bytes lie relative to the block's first key (in elements)
+  const unsigned koff0 = (unsigned)(8 * (c >> 2) + (c & 3)) * HD + g * 8;   // tile 1: + 4 keys
+  const unsigned voff0 = (unsigned)c * page_size + 8 * g;
+  auto load_block = [&](int kb, Block& blk) __attribute__((always_inline)) {
     const int key0 = kb << 5;
+    if (PM == 2) {
+      // the whole block lies in page pgn[0].  Keys at or beyond the end of the context are read as
+      // they lie in the page (it is the request's own) and masked afterwards.
+      const int inpage = key0 & (page_size - 1);
+      const bf16_t* kbase = k_pages + (size_t)pgn[0] * k_page_stride + ((size_t)hk * page_size + inpage) * HD;
+      const bf16_t* vbase = v_pages + (size_t)pgn[0] * k_page_stride + (size_t)hk * HD * page_size + inpage;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+          blk.kf[t][dc].u = make_uint4(0, 0, 0, 0);
+          if (dc * 32 + g * 8 < HD)
+            blk.kf[t][dc].u = *reinterpret_cast<const uint4*>(kbase + (koff0 + t * 4 * HD + dc * 32));
+        }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        blk.vf[dt].u = *reinterpret_cast<const uint4*>(vbase + (voff0 + (unsigned)(dt * 16) * page_size));
+      prefetch_pages(kb + 1);
+      return;
+    }
     int pg[4] = {pgn[0], pgn[1], pgn[2], pgn[3]};
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int ko = 8 * (c >> 2) + 4 * t + (c & 3);
       const int kk = min(key0 + ko, ctx - 1);
       int page, off;
-      if (POW2) {
-        page = pick(pg, page_shift >= 5 ? 0 : (ko >> page_shift));
+      if (PM == 1) {
+        page = pick(pg, ko >> page_shift);
         off = kk & (page_size - 1);
       } else {
         locate(kk, page, off);
@@ -178,7 +224,7 @@ __device__ __forceinline__ void attention_tile(
     }
     if (wide_v) {
       const int run = min(key0 + 8 * g, (ctx - 1) & ~7);
-      const int page = pick(pg, page_shift >= 5 ? 0 : ((8 * g) >> page_shift));
+      const int page = pick(pg, (8 * g) >> page_shift);
       const int off = run & (page_size - 1);
       const bf16_t* vp = v_pages + (size_t)page * k_page_stride + (size_t)hk * HD * page_size + off;
 #pragma unroll
@@ -199,10 +245,11 @@ __device__ __forceinline__ void attention_tile(
     prefetch_pages(kb + 1);
   };
 
-  auto compute = [&](int kb, Block& blk) {
+  // MASKED: some key of the block is invisible to some row (the causal edge, the window's edge,
+  // the end of the context); otherwise no comparison is made at all
+  auto compute = [&](int kb, Block& blk, auto masked) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked)::value;
     const int key0 = kb << 5;
-    // every key of the block visible to every row of the tile: no masking needed
-    const bool full = (key0 + 31 <= ctx_before + j_lo) && (window <= 0 || key0 > ctx_before + j_hi - window);
 
     // ---- S^T = K Q^T --------------------------------------------------------------------
     floatx4_t s[2][NT];
@@ -216,7 +263,7 @@ __device__ __forceinline__ void attention_tile(
           s[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[t][dc].v, qf[n][dc].v, s[t][n], 0, 0, 0);
       }
 
-    if (!full) {
+    if (MASKED) {
       // keys at or beyond the end of the context hold whatever the page held before: their
       // probability is 0, and 0 times such a value must stay 0
       const int first = key0 + 8 * g;
@@ -246,7 +293,7 @@ __device__ __forceinline__ void attention_tile(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float x = s[t][n][r];
-          if (!full) {
+          if (MASKED) {
             const int key = key0 + 8 * g + 4 * t + r;
             const bool vis = key <= qpos[n] && (window <= 0 || key > qpos[n] - window);
             x = vis ? x : -INFINITY;
@@ -254,10 +301,10 @@ __device__ __forceinline__ void attention_tile(
           v[t][r] = x;
           mx = fmaxf(mx, x);
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_across_groups(mx);
       const float m_new = fmaxf(m[n], mx * scale_log2e);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      // a row that has seen no visible key yet keeps m = -inf; only masked blocks can do that
+      const float m_safe = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m[n] - m_safe);
       m[n] = m_new;
       float ps = 0.f;
@@ -286,21 +333,36 @@ __device__ __forceinline__ void attention_tile(
         acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
   };
 
-  // three buffers in turn: the loads of the next two blocks are in flight while one is computed
-  Block buf_a, buf_b, buf_c;
-  prefetch_pages(b0);
-  if (b0 < b1) load_block(b0, buf_a);
-  if (b0 + 1 < b1) load_block(b0 + 1, buf_b);
-  for (int kb = b0; kb < b1; kb += 3) {
-    if (kb + 2 < b1) load_block(kb + 2, buf_c);
-    compute(kb, buf_a);
-    if (kb + 1 < b1) {
-      if (kb + 3 < b1) load_block(kb + 3, buf_a);
-      compute(kb + 1, buf_b);
+  // Three buffers in turn: the loads of the next two blocks are in flight while one is computed.
+  // The loads carry no conditions: a block beyond the last is read from clamped keys and pages and
+  // never used.  With a branch around them the compiler no longer knows how many loads are in
+  // flight where a block's data is awaited, and waits for all of them, the newest included.
+  if (b0 < b1) {
+    Block buf_a, buf_b, buf_c;
+    prefetch_pages(b0);
+    load_block(b0, buf_a);
+    load_block(b0 + 1, buf_b);
+    int kb = b0;
+    for (; kb + 3 <= b1; kb += 3) {
+      if (kb >= full_lo && kb + 2 <= full_hi) {
+        load_block(kb + 2, buf_c);
+        compute(kb, buf_a, Unmasked{});
+        load_block(kb + 3, buf_a);
+        compute(kb + 1, buf_b, Unmasked{});
+        load_block(kb + 4, buf_b);
+        compute(kb + 2, buf_c, Unmasked{});
+      } else {
+        load_block(kb + 2, buf_c);
+        compute(kb, buf_a, Masked{});
+        load_block(kb + 3, buf_a);
+        compute(kb + 1, buf_b, Masked{});
+        load_block(kb + 4, buf_b);
+        compute(kb + 2, buf_c, Masked{});
+      }
     }
-    if (kb + 2 < b1) {
-      if (kb + 4 < b1) load_block(kb + 4, buf_b);
-      compute(kb + 2, buf_c);
+    if (kb < b1) {
+      compute(kb, buf_a, Masked{});
+      if (kb + 1 < b1) compute(kb + 1, buf_b, Masked{});
     }
   }
 
@@ -339,7 +401,7 @@ __device__ __forceinline__ void attention_tile(
 // A wave takes tile w of its (segment, KV head).  With PAIR it takes tile ntiles-1-w as well: under
 // the causal mask tile t reads keys up to about t's end, so the two together are always one full
 // context long and all waves of a prompt finish at about the same time.
-template <int NT, bool POW2, bool PAIR>
+template <int NT, int PM, bool PAIR>
 __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
@@ -353,19 +415,19 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int q_begin = cu_q[seg];
   const int q_len = cu_q[seg + 1] - q_begin;
   if (!PAIR) {
-    attention_tile<NT, POW2>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+    attention_tile<NT, PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
                              max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
                              part_o, part_ml);
     return;
   }
   const int ntiles = (q_len * (Hq / Hk) + 16 * NT - 1) / (16 * NT);
   if (w >= (ntiles + 1) / 2) return;                                  // the second half is done by pairing
-  attention_tile<NT, POW2>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+  attention_tile<NT, PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
                            max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
                            part_o, part_ml);
   const int other = ntiles - 1 - w;
   if (other > w)
-    attention_tile<NT, POW2>(other, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+    attention_tile<NT, PM>(other, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
                              max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
                              part_o, part_ml);
 }
@@ -439,18 +501,22 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
   }
-#define GO(NT, POW2, PAIR)                                                                             \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT, POW2, PAIR>), grid, block, 0, stream,            \
+#define GO(NT, PM, PAIR)                                                                               \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT, PM, PAIR>), grid, block, 0, stream,              \
                      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages,                 \
                      (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
                      page_shift, scale_log2e, window, num_splits, part_o, part_ml)
-  const bool pow2 = page_shift >= 3;
-  if (small && pow2) GO(1, true, false);
-  else if (small) GO(1, false, false);
-  else if (pair && pow2) GO(NT_PREFILL, true, true);
-  else if (pair) GO(NT_PREFILL, false, true);
-  else if (pow2) GO(NT_PREFILL, true, false);
-  else GO(NT_PREFILL, false, false);
+  const int pm = page_shift >= 5 ? 2 : (page_shift >= 3 ? 1 : 0);
+#define GO3(NT, PAIR)           \
+  do {                          \
+    if (pm == 2) GO(NT, 2, PAIR);      \
+    else if (pm == 1) GO(NT, 1, PAIR); \
+    else GO(NT, 0, PAIR);              \
+  } while (0)
+  if (small) GO3(1, false);
+  else if (pair) GO3(NT_PREFILL, true);
+  else GO3(NT_PREFILL, false);
+#undef GO3
 #undef GO
   SA_LAUNCH_CHECK();
   if (num_splits > 1) {

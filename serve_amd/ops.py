@@ -358,7 +358,8 @@ def mfma_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_strid
 
 def attention_splits(decode_only: bool, num_segments: int, num_kv_heads: int, max_ctx_len: int) -> int:
     """Into how many parts the key range of a decode step is cut so that the chip is filled:
-    about 2048 waves in all, and no part shorter than 128 keys."""
+    about 512 waves in all (more cost more in the merge than they gain), and no part shorter than
+    64 keys."""
     if not decode_only:
         return 1
     # both inputs are rounded up to powers of two, so that a step run eagerly and the same step
@@ -369,8 +370,8 @@ def attention_splits(decode_only: bool, num_segments: int, num_kv_heads: int, ma
     segs = 1
     while segs < num_segments:
         segs *= 2
-    by_length = max(1, ctx // 128)
-    by_waves = max(1, 2048 // (segs * num_kv_heads))
+    by_length = max(1, ctx // 64)
+    by_waves = max(1, 512 // (segs * num_kv_heads))
     return max(1, min(by_length, by_waves, 64))
 
 

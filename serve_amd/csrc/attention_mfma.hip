@@ -467,14 +467,15 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
 
 extern "C" int sa_attention_mfma_head_dim() { return HD; }
 
-// tiles of 16*nt rows per wave: nt = 1 for decode-only steps, NT_PREFILL otherwise
+// Tiles of 16*nt rows per wave: nt = 1 when a segment has at most 16 rows (decode steps).  Prompt
+// portions take the largest tile the registers hold (fewest reads of K and V) when that still gives
+// every SIMD of the chip a wave, and 32 rows otherwise.
 #if HEAD_DIM <= 64
 #define NT_PREFILL 4
 #else
 #define NT_PREFILL 2
 #endif
-
-extern "C" int sa_attention_mfma_rows_per_tile(int decode_only) { return decode_only ? 16 : 16 * NT_PREFILL; }
+constexpr int WAVES_TO_FILL = 1024;     // 256 compute units x 4 SIMDs
 
 extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, const void* k_pages,
                                        const void* v_pages, const int* block_table, int max_pages,
@@ -489,11 +490,15 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   if ((long long)B * num_splits > 65535 || Hk > 65535) return SA_ERR_ARG;
   const int G = Hq / Hk;
   const bool small = (long long)max_q_len * G <= 16;
-  const int rows_per_tile = small ? 16 : 16 * NT_PREFILL;
-  const int tiles = (int)(((long long)max_q_len * G + rows_per_tile - 1) / rows_per_tile);
   // prompt portions: a wave takes tiles w and tiles-1-w, so half as many waves are launched
   const bool pair = !small && num_splits == 1;
-  const int waves = pair ? (tiles + 1) / 2 : tiles;
+  int nt = small ? 1 : NT_PREFILL;
+  auto waves_for = [&](int n) {
+    const long long tiles = ((long long)max_q_len * G + 16 * n - 1) / (16 * n);
+    return pair ? (tiles + 1) / 2 : tiles;
+  };
+  if (nt > 2 && waves_for(nt) * Hk * B < WAVES_TO_FILL) nt = 2;
+  const int waves = (int)waves_for(nt);
   dim3 grid((waves + 3) / 4, Hk, B * num_splits), block(256);
   const float scale_log2e = scale * 1.4426950408889634f;
   int page_shift = -1;
@@ -514,8 +519,12 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
     else GO(NT, 0, PAIR);              \
   } while (0)
   if (small) GO3(1, false);
+  else if (nt == 2 && pair) GO3(2, true);
+  else if (nt == 2) GO3(2, false);
+#if NT_PREFILL > 2
   else if (pair) GO3(NT_PREFILL, true);
   else GO3(NT_PREFILL, false);
+#endif
 #undef GO3
 #undef GO
   SA_LAUNCH_CHECK();

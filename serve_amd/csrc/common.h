@@ -69,6 +69,21 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
+// sin and cos of an angle of up to about 2e5 rad (a position times a frequency of at most 1), to
+// about 1e-6: the library's sincosf spends over a thousand cycles on arguments this large.  The
+// multiple of 2 pi is taken off in three steps whose constants have few enough bits for the first
+// products to be exact (6.28125 = 201/32; 2029/2^20; the rest), the remainder goes to the
+// hardware's sine and cosine, which take their argument in turns.
+__device__ __forceinline__ void sincos_reduced(float x, float* sn, float* cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.28125f, x);
+  r = fmaf(-k, 1.93500518798828125e-3f, r);
+  r = fmaf(-k, 3.0199159776e-7f, r);
+  const float t = r * 0.15915494309189535f;
+  *sn = __builtin_amdgcn_sinf(t);
+  *cs = __builtin_amdgcn_cosf(t);
+}
+
 #define SA_LAUNCH_CHECK()                      \
   do {                                         \
     hipError_t e__ = hipGetLastError();        \

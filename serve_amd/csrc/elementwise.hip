@@ -87,7 +87,10 @@ __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = u;
 }
 
-template <typename TA, typename TD, typename TW>
+// PMAX: upper bound of `parts` (1, 4 or 8).  All loads of a thread are issued before anything is
+// added, without conditions around them: a group beyond the row and a part beyond `parts` are read
+// from a clamped address and dropped, so that a row costs one trip to memory and not one per part.
+template <typename TA, typename TD, typename TW, int PMAX>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                                               int parts, size_t part_stride,
                                                               const TW* __restrict__ w, TA* __restrict__ y,
@@ -98,20 +101,28 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   float* xr = x + (size_t)t * d;
   const TD* dr = delta ? delta + (size_t)t * d : nullptr;
   const int groups = d >> 2;
+  const int nk = (groups + 255) >> 8;            // rounds of 256 groups, at most 8
   float4 v[8], wv[8];
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
-    const int i = (threadIdx.x + k * 256) * 4;
-    if (threadIdx.x + k * 256 < groups) {
+    if (k < nk) {
+      const int gi = threadIdx.x + k * 256;
+      const int i = min(gi, groups - 1) * 4;
       v[k] = load4(xr + i);
       wv[k] = load4(w + i);
-      if (dr)
-        for (int p = 0; p < parts; ++p) {
-          const float4 a = load4(dr + p * part_stride + i);
-          v[k].x += a.x; v[k].y += a.y; v[k].z += a.z; v[k].w += a.w;
+      if (dr) {
+        float4 a[PMAX];
+#pragma unroll
+        for (int p = 0; p < PMAX; ++p) a[p] = load4(dr + (size_t)min(p, parts - 1) * part_stride + i);
+#pragma unroll
+        for (int p = 0; p < PMAX; ++p) {
+          const float on = p < parts ? 1.f : 0.f;
+          v[k].x += on * a[p].x; v[k].y += on * a[p].y; v[k].z += on * a[p].z; v[k].w += on * a[p].w;
         }
-      ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+      }
+      const float in = gi < groups ? 1.f : 0.f;
+      ss += in * (v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w);
     }
   }
   ss = block_sum(ss, scratch);
@@ -119,8 +130,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   TA* yr = y + (size_t)r * d;
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
-    const int i = (threadIdx.x + k * 256) * 4;
-    if (threadIdx.x + k * 256 < groups) {
+    const int gi = threadIdx.x + k * 256;
+    const int i = gi * 4;
+    if (k < nk && gi < groups) {
       if (dr && !rows) store4(xr + i, v[k]);
       store4(yr + i, make_float4((v[k].x * rs) * wv[k].x, (v[k].y * rs) * wv[k].y,
                                  (v[k].z * rs) * wv[k].z, (v[k].w * rs) * wv[k].w));
@@ -142,8 +154,14 @@ extern "C" int sa_add_rmsnorm(float* x, const void* delta, int delta_dtype, int 
   dim3 grid(R), block(vec || d >= 1024 ? 256 : 64);
 #define GO(TA, TD, TW)                                                                                   \
   do {                                                                                                   \
-    if (vec)                                                                                             \
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TD, TW>), grid, block, 0, stream, x,                \
+    if (vec && parts == 1)                                                                               \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TD, TW, 1>), grid, block, 0, stream, x,             \
+                         (const TD*)delta, parts, part_stride, (const TW*)w, (TA*)y, rows, eps, d);      \
+    else if (vec && parts <= 4)                                                                          \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TD, TW, 4>), grid, block, 0, stream, x,             \
+                         (const TD*)delta, parts, part_stride, (const TW*)w, (TA*)y, rows, eps, d);      \
+    else if (vec && parts <= 8)                                                                          \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TD, TW, 8>), grid, block, 0, stream, x,             \
                          (const TD*)delta, parts, part_stride, (const TW*)w, (TA*)y, rows, eps, d);      \
     else                                                                                                 \
       hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TD, TW>), grid, block, 0, stream, x, (const TD*)delta,  \
@@ -190,7 +208,8 @@ __global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict
     const int i0 = adjacent ? 2 * j : j;
     const int i1 = adjacent ? 2 * j + 1 : j + half;
     float sn, cs;
-    sincosf(pos * inv_freq[j], &sn, &cs);
+    if (sizeof(TA) == 2) sincos_reduced(pos * inv_freq[j], &sn, &cs);   // bf16 keeps 8 bits of it
+    else sincosf(pos * inv_freq[j], &sn, &cs);
     TA* hp = row + (size_t)h * D;
     const float a = to_float(hp[i0]);
     const float b = to_float(hp[i1]);

@@ -29,7 +29,6 @@ union Frag {
 // KU = k-chunks of 32 loaded before their products are issued (loads in flight per wave).
 // gridDim.z > 1 cuts K across workgroups as well: workgroup z writes its partial sums to
 // C + z * M * N (fp32), and the consumer adds the parts in order.
-// STREAM: weights are loaded with the non-temporal hint (they are read once per step).
 // EPI selects what is done with the sums: EPI_PLAIN stores them; EPI_SWIGLU pairs gate row n with up
 // row I + n and stores silu(gate) * up; EPI_QKV_ROPE pairs row j of a head with row j + D/2 of the
 // same head of the stacked q/k/v matrix, rotates the q and k pairs by position (the rotation of
@@ -45,21 +44,6 @@ struct QkvRopeArgs {
   bf16_t* v_pages;          // [P, Hk, D, page_size]
   int Hq, Hk, D, page_size;
 };
-
-// sin and cos of an angle of up to about 2e5 rad (a position times a frequency of at most 1), to
-// about 1e-6: the library's sincosf spends over a thousand cycles on arguments this large.  The
-// multiple of 2 pi is taken off in three steps whose constants have few enough bits for the first
-// products to be exact (6.28125 = 201/32; 2029/2^20; the rest), the remainder goes to the
-// hardware's sine and cosine, which take their argument in turns.
-__device__ __forceinline__ void sincos_reduced(float x, float* sn, float* cs) {
-  const float k = rintf(x * 0.15915494309189535f);
-  float r = fmaf(-k, 6.28125f, x);
-  r = fmaf(-k, 1.93500518798828125e-3f, r);
-  r = fmaf(-k, 3.0199159776e-7f, r);
-  const float t = r * 0.15915494309189535f;
-  *sn = __builtin_amdgcn_sinf(t);
-  *cs = __builtin_amdgcn_cosf(t);
-}
 
 // What is done with a wave's finished sums acc[rt][mt] (lane l: activation row m0 + 16 mt + l%16,
 // outputs 4*(l/16) .. +3 of row tile rt); the row tiles start at n0 as the kernels below lay them out.
@@ -144,7 +128,7 @@ __device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __rest
   }
 }
 
-template <int RT, int MT, int KS, int KU, typename TC, int EPI, bool STREAM = false>
+template <int RT, int MT, int KS, int KU, typename TC, int EPI>
 __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                              const bf16_t* __restrict__ W,
                                                              TC* __restrict__ C, int M, int N, int K,
@@ -175,24 +159,25 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   const int ch_end = min(wg_end, ch_begin + per);
   C += (size_t)blockIdx.z * M * N;
 
+  // Loads carry no per-lane conditions (a branch around every load would serialize them): rows
+  // beyond M or N are read from row 0 and give sums that are never stored; beyond the wave's slice
+  // of K the address is clamped and the activation operand is zeroed, which zeroes the product
+  // whatever finite weight stands there.
   const bf16_t* wrow[RT];
-  bool wok[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     int n;
     if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
     else if (QKV) n = n0 + rt * (qa.D >> 1) + c;
     else n = n0 + rt * 16 + c;
-    wok[rt] = SWIGLU ? (n0 + c < N) : (n < N);
-    wrow[rt] = W + (size_t)(wok[rt] ? n : 0) * K;
+    const bool ok = SWIGLU ? (n0 + c < N) : (n < N);
+    wrow[rt] = W + (size_t)(ok ? n : 0) * K;
   }
   const bf16_t* arow[MT];
-  bool aok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = m0 + mt * 16 + c;
-    aok[mt] = m < M;
-    arow[mt] = A + (size_t)(aok[mt] ? m : 0) * K;
+    arow[mt] = A + (size_t)(m < M ? m : 0) * K;
   }
 
   floatx4_t acc[RT][MT];
@@ -201,30 +186,23 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
 
-  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
   for (int ch = ch_begin; ch < ch_end; ch += KU) {
     Frag wf[RT][KU], af[MT][KU];
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
-      const int k = (ch + u) * 32 + g * 8;
-      const bool kin = (ch + u) < ch_end && k < K;
+      const int k = min((ch + u) * 32 + g * 8, K - 8);
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        wf[rt][u].u = zero;
-        if (kin && wok[rt]) {
-          const uint4* src = reinterpret_cast<const uint4*>(wrow[rt] + k);
-          if (STREAM) {
-            const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
-            wf[rt][u].u = make_uint4(t.x, t.y, t.z, t.w);
-          } else {
-            wf[rt][u].u = *src;
-          }
-        }
-      }
+      for (int rt = 0; rt < RT; ++rt) wf[rt][u].r = *reinterpret_cast<const u32x4_t*>(wrow[rt] + k);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        af[mt][u].u = zero;
-        if (kin && aok[mt]) af[mt][u].u = *reinterpret_cast<const uint4*>(arow[mt] + k);
+      for (int mt = 0; mt < MT; ++mt) af[mt][u].r = *reinterpret_cast<const u32x4_t*>(arow[mt] + k);
+    }
+    if (ch + KU > ch_end || (ch + KU) * 32 > K) {          // the last, partial round of the slice
+#pragma unroll
+      for (int u = 0; u < KU; ++u) {
+        const bool kin = (ch + u) < ch_end && (ch + u) * 32 + g * 8 < K;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) af[mt][u].r = kin ? af[mt][u].r : zero;
       }
     }
 #pragma unroll

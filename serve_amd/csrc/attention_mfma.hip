@@ -434,13 +434,25 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 
 // out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s; at most 64 splits.
 // One wave per (token, head): the lanes first share the work over the splits (weights), then over
-// the head dims (weighted sum, with independent loads that can all be in flight).
+// the head dims (weighted sum).  S: upper bound of the number of splits; the partial outputs are
+// loaded (all at once, no conditions: a split beyond the last is read from the last and weighs 0)
+// before the weights are known, so that the kernel costs one trip to memory and not two.
+template <int S>
 __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o,
                                                           const float* __restrict__ part_ml,
                                                           bf16_t* __restrict__ out, int num_splits) {
   __shared__ float wgt[64];
   const size_t item = blockIdx.x;                 // token * Hq + head
   const int lane = threadIdx.x;
+  constexpr int NA = (HD + 63) / 64;
+  const float* po = part_o + item * num_splits * HD;
+  float o[NA][S];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) {
+    const int d = min(lane + a * 64, HD - 1);
+#pragma unroll
+    for (int s = 0; s < S; ++s) o[a][s] = po[(size_t)min(s, num_splits - 1) * HD + d];
+  }
   float ms = -INFINITY, ls = 0.f;
   if (lane < num_splits) {
     ms = part_ml[(item * num_splits + lane) * 2];
@@ -452,16 +464,13 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
   wgt[lane] = w;
   __syncthreads();
   const float inv = 1.f / L;
-  const float* po = part_o + item * num_splits * HD;
 #pragma unroll
-  for (int a = 0; a < (HD + 63) / 64; ++a) {
+  for (int a = 0; a < NA; ++a) {
     const int d = lane + a * 64;
-    if (d < HD) {
-      float o = 0.f;
-#pragma unroll 8
-      for (int s = 0; s < num_splits; ++s) o += po[(size_t)s * HD + d] * wgt[s];
-      out[item * HD + d] = from_float<bf16_t>(o * inv);
-    }
+    float sum = 0.f;
+#pragma unroll
+    for (int s = 0; s < S; ++s) sum += o[a][s] * wgt[s];
+    if (d < HD) out[item * HD + d] = from_float<bf16_t>(sum * inv);
   }
 }
 
@@ -529,8 +538,15 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
 #undef GO
   SA_LAUNCH_CHECK();
   if (num_splits > 1) {
-    hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml,
-                       (bf16_t*)out, num_splits);
+#define MERGE(S)                                                                                      \
+  hipLaunchKernelGGL(merge_splits_kernel<S>, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml, \
+                     (bf16_t*)out, num_splits)
+    if (num_splits <= 4) MERGE(4);
+    else if (num_splits <= 8) MERGE(8);
+    else if (num_splits <= 16) MERGE(16);
+    else if (num_splits <= 32) MERGE(32);
+    else MERGE(64);
+#undef MERGE
     SA_LAUNCH_CHECK();
   }
   return 0;

@@ -30,10 +30,12 @@ union Frag {
 // gridDim.z > 1 cuts K across workgroups as well: workgroup z writes its partial sums to
 // C + z * M * N (fp32), and the consumer adds the parts in order.
 // EPI selects what is done with the sums: EPI_PLAIN stores them; EPI_SWIGLU pairs gate row n with up
-// row I + n and stores silu(gate) * up; EPI_QKV_ROPE pairs row j of a head with row j + D/2 of the
-// same head of the stacked q/k/v matrix, rotates the q and k pairs by position (the rotation of
-// serve/model.py:234-244 on the checkpoint's row order) and stores q to its buffer and k and v
-// straight into the cache pages of each token's slot (serve/kernels/cache_write.py:49-165).
+// row I + n and stores silu(gate) * up; EPI_QKV_ROPE works on one tile of 16 rows of the stacked
+// q/k/v matrix that holds eight dims j.. of a head and their partners j + D/2..: the sums of a pair
+// sit in lanes 32 apart and are exchanged with one row swap each, the q and k pairs are rotated by
+// position (the rotation of serve/model.py:234-244 on the checkpoint's row order), q goes to its
+// buffer and k and v straight into the cache pages of each token's slot
+// (serve/kernels/cache_write.py:49-165).
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_QKV_ROPE = 2 };
 
 struct QkvRopeArgs {
@@ -45,11 +47,60 @@ struct QkvRopeArgs {
   int Hq, Hk, D, page_size;
 };
 
+// What the rotating epilogue needs besides the sums: read when a kernel starts, so that the trip to
+// memory for them runs beside the product and not after it.
+template <int MT>
+struct QkvLane {
+  float pos[MT];
+  int slot[MT];
+  float freq[4];
+};
+
+template <int MT>
+__device__ __forceinline__ QkvLane<MT> load_qkv_lane(const QkvRopeArgs& qa, int M, int m0, int head, int t8,
+                                                     int g, int c) {
+  QkvLane<MT> ql;
+  const bool rotated = head < qa.Hq + qa.Hk;
+  const bool stored = head >= qa.Hq && head < qa.Hq + 2 * qa.Hk;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = min(m0 + mt * 16 + c, M - 1);
+    ql.pos[mt] = rotated ? (float)qa.positions[m] : 0.f;
+    ql.slot[mt] = stored ? qa.slots[m] : -1;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) ql.freq[r] = rotated ? qa.inv_freq[t8 * 8 + 4 * (g & 1) + r] : 0.f;
+  return ql;
+}
+
+__device__ __forceinline__ void store4(float* p, const float (&v)[4], bool vec) {
+  if (vec) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) p[r] = v[r];
+  }
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4], bool vec) {
+  if (vec) {
+    uint2 u;
+    u.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+    u.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) p[r] = from_float<bf16_t>(v[r]);
+  }
+}
+
 // What is done with a wave's finished sums acc[rt][mt] (lane l: activation row m0 + 16 mt + l%16,
-// outputs 4*(l/16) .. +3 of row tile rt); the row tiles start at n0 as the kernels below lay them out.
+// outputs 4*(l/16) .. +3 of row tile rt); the row tiles start at n0 as the kernels below lay them
+// out.  A lane's four outputs are consecutive in memory and go out as one store where the row
+// length keeps them aligned.
 template <int RT, int MT, typename TC, int EPI>
 __device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __restrict__ C, int M, int N, int m0,
-                                            int n0, int head, int t16, const QkvRopeArgs& qa, int g, int c) {
+                                            int n0, int head, int t16, const QkvRopeArgs& qa,
+                                            const QkvLane<MT>& ql, int g, int c) {
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
   constexpr bool QKV = EPI == EPI_QKV_ROPE;
   const int ldc = N;
@@ -58,72 +109,78 @@ __device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __rest
     const int m = m0 + mt * 16 + c;
     if (m >= M) continue;
     if (SWIGLU) {
+      const int n = n0 + 4 * g;
+      float o[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int n = n0 + 4 * g + r;
-        if (n < N) {
-          const float gt = acc[0][mt][r];
-          const float up = acc[1][mt][r];
-          C[(size_t)m * ldc + n] = from_float<TC>((gt / (1.f + __expf(-gt))) * up);
-        }
+        const float gt = acc[0][mt][r];
+        const float up = acc[1][mt][r];
+        o[r] = (gt / (1.f + __expf(-gt))) * up;
+      }
+      if (n + 3 < N) {
+        store4(C + (size_t)m * ldc + n, o, (N & 3) == 0);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) C[(size_t)m * ldc + n + r] = from_float<TC>(o[r]);
       }
     } else if (QKV) {
-      const int D = qa.D, half = qa.D >> 1;
-      const int dim0 = t16 * 16 + 4 * g;                 // this lane's four dims, and dim0 + D/2 ..
-      float lo[4], hi[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        lo[r] = acc[0][mt][r];
-        hi[r] = acc[1][mt][r];
-      }
-      if (head < qa.Hq + qa.Hk) {
-        const float pos = (float)qa.positions[m];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float sn, cs;
-          sincos_reduced(pos * qa.inv_freq[dim0 + r], &sn, &cs);
-          const float a = lo[r], b = hi[r];
-          lo[r] = a * cs - b * sn;
-          hi[r] = b * cs + a * sn;
-        }
-      }
-      if (head < qa.Hq) {
-        TC* qp = C + ((size_t)m * qa.Hq + head) * D + dim0;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          qp[r] = from_float<TC>(lo[r]);
-          qp[half + r] = from_float<TC>(hi[r]);
-        }
-      } else {
-        const int slot = qa.slots[m];
-        if (slot >= 0) {
-          const int page = slot / qa.page_size;
-          const int off = slot - page * qa.page_size;
-          if (head < qa.Hq + qa.Hk) {
-            bf16_t* kp = qa.k_pages + (((size_t)page * qa.Hk + (head - qa.Hq)) * qa.page_size + off) * D + dim0;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              kp[r] = from_float<bf16_t>(lo[r]);
-              kp[half + r] = from_float<bf16_t>(hi[r]);
-            }
-          } else {
-            bf16_t* vp = qa.v_pages + (((size_t)page * qa.Hk + (head - qa.Hq - qa.Hk)) * D + dim0) * qa.page_size + off;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              vp[(size_t)r * qa.page_size] = from_float<bf16_t>(lo[r]);
-              vp[(size_t)(half + r) * qa.page_size] = from_float<bf16_t>(hi[r]);
-            }
-          }
-        }
-      }
+      // handled below, outside this loop's early exit: the exchange needs both partner lanes
     } else {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+      for (int rt = 0; rt < RT; ++rt) {
+        const int n = n0 + rt * 16 + 4 * g;
+        float o[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int n = n0 + rt * 16 + 4 * g + r;
-          if (n < N) C[(size_t)m * ldc + n] = from_float<TC>(acc[rt][mt][r]);
+        for (int r = 0; r < 4; ++r) o[r] = acc[rt][mt][r];
+        if (n + 3 < N) {
+          store4(C + (size_t)m * ldc + n, o, (N & 3) == 0);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < N) C[(size_t)m * ldc + n + r] = from_float<TC>(o[r]);
         }
+      }
+    }
+  }
+  if (QKV) {
+    // rows 0..7 of the tile are dims d0.. of the head, rows 8..15 their partners d0 + D/2..; lane
+    // groups 0, 1 hold the former, 2, 3 the latter, for the same activation row: lanes 32 apart
+    const int D = qa.D, half = qa.D >> 1;
+    const bool upper = g >= 2;
+    const int dim0 = t16 * 8 + 4 * (g & 1) + (upper ? half : 0);     // this lane's four consecutive dims
+    const bool rotated = head < qa.Hq + qa.Hk;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = m0 + mt * 16 + c;
+      float o[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float own = acc[0][mt][r];
+        const uint32_t u = __float_as_uint(own);
+        const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        const float partner = __uint_as_float(upper ? sw[0] : sw[1]);
+        float sn, cs;
+        sincos_reduced(ql.pos[mt] * ql.freq[r], &sn, &cs);
+        // lower: a cos - b sin with a = own; upper: b cos + a sin with b = own
+        o[r] = rotated ? (upper ? own * cs + partner * sn : own * cs - partner * sn) : own;
+      }
+      if (m >= M) continue;
+      if (head < qa.Hq) {
+        store4(C + ((size_t)m * qa.Hq + head) * D + dim0, o, true);      // D % 16 == 0: 8-byte aligned
+      } else {
+        const int slot = ql.slot[mt];
+        if (slot < 0) continue;
+        const int page = slot / qa.page_size;
+        const int off = slot - page * qa.page_size;
+        if (head < qa.Hq + qa.Hk) {
+          store4(qa.k_pages + (((size_t)page * qa.Hk + (head - qa.Hq)) * qa.page_size + off) * D + dim0, o, true);
+        } else {
+          bf16_t* vp = qa.v_pages + (((size_t)page * qa.Hk + (head - qa.Hq - qa.Hk)) * D + dim0) * qa.page_size + off;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) vp[(size_t)r * qa.page_size] = from_float<bf16_t>(o[r]);
+        }
+      }
     }
   }
 }
@@ -136,19 +193,24 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
   constexpr bool QKV = EPI == EPI_QKV_ROPE;
   static_assert(KS * RT * MT <= 64, "partial sums must fit into 64 KB of LDS");
-  static_assert(EPI == EPI_PLAIN || RT == 2, "the pairing epilogues work on two row tiles");
+  static_assert(EPI != EPI_SWIGLU || RT == 2, "gate and up rows are two row tiles");
+  static_assert(EPI != EPI_QKV_ROPE || RT == 1, "a pair of dims sits in one row tile");
   __shared__ float red[KS][RT * MT * 4][64];
 
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
   const int c = lane & 15;
-  // first row of this workgroup's (first) tile; QKV: tile t16 of head `head`, second tile D/2 below
-  const int tph = QKV ? (qa.D >> 5) : 1;
+  // first row of this workgroup's (first) tile; QKV: tile t16 of head `head` = its dims 8 t16 .. + 7
+  // and their partners D/2 further on
+  const int tph = QKV ? (qa.D >> 4) : 1;
   const int head = QKV ? blockIdx.x / tph : 0;
   const int t16 = QKV ? blockIdx.x - head * tph : 0;
-  const int n0 = QKV ? head * qa.D + t16 * 16 : blockIdx.x * (SWIGLU ? 16 : RT * 16);
+  const int n0 = QKV ? head * qa.D + t16 * 8 : blockIdx.x * (SWIGLU ? 16 : RT * 16);
   const int m0 = blockIdx.y * (MT * 16);
+
+  QkvLane<MT> ql = {};
+  if (QKV) ql = load_qkv_lane<MT>(qa, M, m0, head, t16, g, c);
 
   const int nchunks = (K + 31) >> 5;
   const int per_wg = (nchunks + gridDim.z - 1) / gridDim.z;
@@ -168,7 +230,7 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   for (int rt = 0; rt < RT; ++rt) {
     int n;
     if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
-    else if (QKV) n = n0 + rt * (qa.D >> 1) + c;
+    else if (QKV) n = n0 + (c < 8 ? c : (qa.D >> 1) + c - 8);
     else n = n0 + rt * 16 + c;
     const bool ok = SWIGLU ? (n0 + c < N) : (n < N);
     wrow[rt] = W + (size_t)(ok ? n : 0) * K;
@@ -236,7 +298,7 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
         }
   }
 
-  store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, g, c);
+  store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, ql, g, c);
 }
 
 // The same products for 17..64 rows of activations (decode at larger batches, short prompt
@@ -256,7 +318,8 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
                                                                 int up_offset, QkvRopeArgs qa) {
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
   constexpr bool QKV = EPI == EPI_QKV_ROPE;
-  static_assert(EPI == EPI_PLAIN || RT == 2, "the pairing epilogues work on two row tiles");
+  static_assert(EPI != EPI_SWIGLU || RT == 2, "gate and up rows are two row tiles");
+  static_assert(EPI != EPI_QKV_ROPE || RT == 1, "a pair of dims sits in one row tile");
   static_assert(KH == 2 || KH == 4 || KH == 8, "a stage is 8 steps of 32");
   constexpr int THREADS = 64 * NR * KH;
   constexpr int ROWS = MT * 16;            // activation rows of a workgroup
@@ -274,11 +337,14 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
   const int rg = wave % NR;                // row group
   const int kh = wave / NR;                // K slice
   const int tile = blockIdx.x * NR + rg;
-  const int tph = QKV ? (qa.D >> 5) : 1;
+  const int tph = QKV ? (qa.D >> 4) : 1;
   const int head = QKV ? tile / tph : 0;
   const int t16 = QKV ? tile - head * tph : 0;
-  const int n0 = QKV ? head * qa.D + t16 * 16 : tile * (SWIGLU ? 16 : RT * 16);
+  const int n0 = QKV ? head * qa.D + t16 * 8 : tile * (SWIGLU ? 16 : RT * 16);
   const int m0 = blockIdx.y * ROWS;
+
+  QkvLane<MT> ql = {};
+  if (QKV) ql = load_qkv_lane<MT>(qa, M, m0, head, t16, g, c);
 
   // this workgroup's slice of K, in chunks of 32
   const int nchunks = (K + 31) >> 5;
@@ -303,7 +369,7 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
   for (int rt = 0; rt < RT; ++rt) {
     int n;
     if (SWIGLU) n = (rt == 0 ? 0 : up_offset) + n0 + c;
-    else if (QKV) n = n0 + rt * (qa.D >> 1) + c;
+    else if (QKV) n = n0 + (c < 8 ? c : (qa.D >> 1) + c - 8);
     else n = n0 + rt * 16 + c;
     bool ok = SWIGLU ? (n0 + c < N) : (n < N);
     if (QKV) ok = head < qa.Hq + 2 * qa.Hk;
@@ -425,7 +491,7 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
         acc[rt][mt][r] = sum;
       }
   if (QKV && head >= qa.Hq + 2 * qa.Hk) return;
-  store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, g, c);
+  store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, ql, g, c);
 }
 
 template <int RT, int MT, int NR, int KH, typename TC, int EPI>
@@ -433,7 +499,7 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
                       const QkvRopeArgs& qa, hipStream_t stream) {
   unsigned tiles;
   if (EPI == EPI_SWIGLU) tiles = (N + 15) / 16;
-  else if (EPI == EPI_QKV_ROPE) tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 5);
+  else if (EPI == EPI_QKV_ROPE) tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
   else tiles = (N + RT * 16 - 1) / (RT * 16);
   dim3 grid((tiles + NR - 1) / NR, (M + MT * 16 - 1) / (MT * 16), parts);
   if (grid.y > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
@@ -457,12 +523,14 @@ static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, 
     if (four) GO(2, 4, 4, 2);        // many: 128 a workgroup, which halves the activation traffic
     GO(2, 2, 4, 2);
   }
-  if constexpr (EPI == EPI_QKV_ROPE) {  // few rows again: one pair of tiles a workgroup, K cut eight ways
-    if (four) GO(2, 4, 1, 8);
-    GO(2, 2, 1, 8);
+  if constexpr (EPI == EPI_QKV_ROPE) {  // few rows again: one tile a workgroup, K cut eight ways
+    if (four) GO(1, 4, 1, 8);
+    GO(1, 2, 1, 8);
   }
-  if (four) GO(2, 4, 2, 4);
-  GO(2, 2, 2, 4);
+  if constexpr (EPI == EPI_SWIGLU) {
+    if (four) GO(2, 4, 2, 4);
+    GO(2, 2, 2, 4);
+  }
 #undef GO
   return SA_ERR_ARG;
 }
@@ -472,7 +540,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int M, int N, in
                          int parts, const QkvRopeArgs& qa, hipStream_t stream) {
   unsigned gx;
   if (EPI == EPI_SWIGLU) gx = (N + 15) / 16;
-  else if (EPI == EPI_QKV_ROPE) gx = (qa.Hq + 2 * qa.Hk) * (qa.D >> 5);
+  else if (EPI == EPI_QKV_ROPE) gx = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
   else gx = (N + RT * 16 - 1) / (RT * 16);
   dim3 grid(gx, (M + MT * 16 - 1) / (MT * 16), parts);
   if (grid.y > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
@@ -487,13 +555,14 @@ static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int 
                        int parts, const QkvRopeArgs& qa, hipStream_t stream) {
   // up to 16 rows of activations (more take the kernel above; still more would loop over grid.y).
   // Many weight rows: 2 row tiles per wave and few waves; few rows: more waves splitting K.
-  const bool wide = EPI == EPI_SWIGLU || N >= 8192;
 #define GO(RT, MT, KS, KU) \
   return launch_skinny<RT, MT, KS, KU, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
-  // (the choices below are the best of a sweep over RT, KS and KU at the Llama-3.2-1B sizes)
-  if constexpr (EPI == EPI_QKV_ROPE) GO(2, 1, 8, 8);
-  if (wide) GO(2, 1, 2, 8);
+  // (the choices below are the best of a sweep over RT, KS and KU at the Llama-3.2-1B sizes; the
+  // sweep is flat: every shape that fills the chip runs at about 3 us + bytes / 5.3 TB/s)
+  if constexpr (EPI == EPI_QKV_ROPE) GO(1, 1, 8, 8);
+  if constexpr (EPI == EPI_SWIGLU) GO(2, 1, 2, 8);
   if constexpr (EPI == EPI_PLAIN) {
+    if (N >= 8192) GO(2, 1, 2, 8);
     if (parts > 1) GO(1, 1, 2, 8);   // K is already cut across workgroups: 2 waves each
     GO(1, 1, 16, 4);
   }
@@ -530,12 +599,12 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
 
 // q, k, v = A [Wq; Wk; Wv]^T with W stacked as [(Hq + 2 Hk) D, K]; q and k rotated by position
 // (pairs (j, j + D/2), all D dims); q goes to Q [M, Hq D], k and v into the cache pages.
-// Needs D % 32 == 0.
+// Needs D % 16 == 0.
 extern "C" int sa_gemm_bf16_qkv_rope(const void* A, const void* W, void* Q, const int* positions,
                                      const float* inv_freq, const int* slots, void* k_pages, void* v_pages,
                                      int M, int K, int Hq, int Hk, int D, int page_size, hipStream_t stream) {
   if (M <= 0) return 0;
-  if (K <= 0 || (K & 7) || Hq <= 0 || Hk <= 0 || D <= 0 || (D & 31) || page_size <= 0) return SA_ERR_ARG;
+  if (K <= 0 || (K & 7) || Hq <= 0 || Hk <= 0 || D <= 0 || (D & 15) || page_size <= 0) return SA_ERR_ARG;
   const QkvRopeArgs qa = {positions, inv_freq, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size};
   if (M > 16) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   return pick_skinny<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);

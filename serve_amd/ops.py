@@ -317,9 +317,9 @@ def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> 
 def qkv_rope_available(a: torch.Tensor, w_qkv: torch.Tensor, k_pages: torch.Tensor, head_dim: int,
                        rot_dim: int, adjacent_pairs: bool) -> bool:
     """Whether projection, rotation and cache write can run as one kernel: bf16, few rows, all
-    dims of a head rotated in (j, j + D/2) pairs, head size a multiple of 32."""
+    dims of a head rotated in (j, j + D/2) pairs, head size a multiple of 16."""
     return (a.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
-            and a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0 and head_dim % 32 == 0
+            and a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0 and head_dim % 16 == 0
             and rot_dim == head_dim and not adjacent_pairs and _aligned16(a, w_qkv))
 
 

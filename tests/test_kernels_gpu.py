@@ -435,7 +435,8 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
 
 
 @pytest.mark.parametrize("M,Hq,Hk,D,ps,d", [(1, 4, 2, 32, 8, 64), (8, 32, 8, 64, 16, 2048), (13, 3, 1, 96, 4, 72),
-                                             (40, 6, 2, 128, 16, 200), (64, 2, 2, 64, 32, 96), (16, 5, 1, 64, 8, 520)])
+                                             (40, 6, 2, 128, 16, 200), (64, 2, 2, 64, 32, 96), (16, 5, 1, 64, 8, 520), (9, 2, 2, 48, 8, 64),
+                                             (33, 3, 1, 80, 16, 104), (5, 4, 4, 16, 4, 40)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
     P = 7
@@ -466,4 +467,4 @@ def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     mask = torch.ones((P, ps), dtype=torch.bool, device=DEV)
     mask[page, off] = False
     assert k1.permute(0, 2, 1, 3)[mask].abs().max().item() == 0 and v1.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
-    assert not ops.qkv_rope_available(h, w, k1, 48, 48, False) and not ops.qkv_rope_available(h, w, k1, D, D, True)
+    assert not ops.qkv_rope_available(h, w, k1, 24, 24, False) and not ops.qkv_rope_available(h, w, k1, D, D, True)

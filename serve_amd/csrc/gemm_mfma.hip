@@ -307,8 +307,8 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
 // NR groups of weight rows times KH slices of each 256-wide stage of K; the NR waves of a slice read
 // the same activation fragments, and the KH slices add their sums through LDS at the end, in order.
 // Weight fragments go from global memory straight into registers, two stages ahead of the products;
-// activations are loaded one stage ahead into registers and written to the LDS buffer of their
-// stage (two buffers in turn: one barrier per stage).  A row of a stage holds 32 segments of
+// activations are loaded two stages ahead into registers as well and written to the LDS buffer of
+// their stage when it begins (two buffers in turn: one barrier per stage).  A row of a stage holds 32 segments of
 // 16 bytes; segment s of row r is stored at slot s ^ (r % 16), which makes both the stores (16 lanes
 // along a row) and the fragment reads (16 lanes along a column of segments) free of bank conflicts.
 template <int RT, int MT, int NR, int KH, typename TC, int EPI>
@@ -400,8 +400,7 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
   // the slice of K the address is clamped and the activation operand is zeroed on its way into LDS,
   // which zeroes the product whatever finite weight stands there.
   const u32x4_t zero = {0u, 0u, 0u, 0u};
-  u32x4_t areg[NA];
-  auto load_acts = [&](int s) __attribute__((always_inline)) {
+  auto load_acts = [&](int s, u32x4_t (&areg)[NA]) __attribute__((always_inline)) {
     const int k0 = stage_k(s);
 #pragma unroll
     for (int j = 0; j < NA; ++j)
@@ -416,22 +415,24 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
       for (int rt = 0; rt < RT; ++rt) wf[rt][u].r = *reinterpret_cast<const u32x4_t*>(wrow[rt] + k);
     }
   };
-  // one stage: publish its activations, start the loads of what comes next (activations one
-  // stage ahead, weights two), multiply
-  auto stage = [&](int s, Frag (&cur)[RT][KU], Frag (&pre)[RT][KU]) __attribute__((always_inline)) {
+  // one stage: publish its activations, start the loads of the stage after the next (both the
+  // latency of L2 for the activations and of HBM for the weights take longer than a stage's
+  // products), multiply
+  auto stage = [&](int s, Frag (&cur)[RT][KU], Frag (&pre)[RT][KU], u32x4_t (&acur)[NA],
+                   u32x4_t (&apre)[NA]) __attribute__((always_inline)) {
     constexpr int BUF = ROWS * 32;                      // 16-byte slots per buffer
     const int b = s & 1;
     const int k0 = stage_k(s);
     if (k0 + 256 > k_end) {          // the zeroing waits for the loads, so it is done here and not where they start
 #pragma unroll
-      for (int j = 0; j < NA; ++j) areg[j] = k0 + aseg[j] * 8 < k_end ? areg[j] : zero;
+      for (int j = 0; j < NA; ++j) acur[j] = k0 + aseg[j] * 8 < k_end ? acur[j] : zero;
     }
 #pragma unroll
-    for (int j = 0; j < NA; ++j) adst[j][b * BUF] = areg[j];
+    for (int j = 0; j < NA; ++j) adst[j][b * BUF] = acur[j];
     __syncthreads();
     // (unconditional, so that the number of loads in flight is known where their results are
     // awaited; past the last stage they read it again and nobody uses them)
-    load_acts(min(s + 1, nstages - 1));
+    load_acts(min(s + 2, nstages - 1), apre);
     load_weights(min(s + 2, nstages - 1), pre);
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
@@ -447,22 +448,24 @@ __global__ __launch_bounds__(64 * NR * KH) void gemm_mid_kernel(const bf16_t* __
   };
 
   Frag w0[RT][KU], w1[RT][KU], w2[RT][KU];
+  u32x4_t a0[NA], a1[NA], a2[NA];
   if (nstages > 0) {
-    load_acts(0);
+    load_acts(0, a0);
     load_weights(0, w0);
+    load_acts(min(1, nstages - 1), a1);
     load_weights(min(1, nstages - 1), w1);
   }
   // three stages a turn so that the register sets take turns without copies; the turn has no
   // branches inside, which keeps the compiler's count of loads in flight exact
   int s = 0;
   for (; s + 3 <= nstages; s += 3) {
-    stage(s, w0, w2);
-    stage(s + 1, w1, w0);
-    stage(s + 2, w2, w1);
+    stage(s, w0, w2, a0, a2);
+    stage(s + 1, w1, w0, a1, a0);
+    stage(s + 2, w2, w1, a2, a1);
   }
   if (s < nstages) {
-    stage(s, w0, w2);
-    if (s + 1 < nstages) stage(s + 1, w1, w0);
+    stage(s, w0, w2, a0, a2);
+    if (s + 1 < nstages) stage(s + 1, w1, w0, a1, a0);
   }
 
   // add the slices of K in a fixed order: the waves of slices 1.. hand their sums over through LDS

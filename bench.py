@@ -156,7 +156,7 @@ def main() -> int:
     step_bytes = weight_bytes(cfg) + args.batch * mean_ctx * kv_bytes_per_token(cfg)
     achieved = step_bytes / (dt / steps)
     out = {
-        "metric": "decode tokens/s, Llama-3.2-1B shape, batch 8, context 4096, one MI355X",
+        "metric": f"decode tokens/s, Llama-3.2-1B shape, batch {args.batch}, context {args.context}, one MI355X",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",

@@ -242,6 +242,69 @@ __global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict
   }
 }
 
+// The same for bf16 with (j, j + D/2) pairs over the whole head (rot_dim == D, D % 16 == 0), 16-byte
+// vectors: a thread takes eight pairs of one head (two loads, two stores), then eight dims of one
+// V head (one load, eight scattered stores into the transposed page).
+__global__ __launch_bounds__(256) void rope_kv_write_bf16_vec_kernel(
+    bf16_t* __restrict__ qkv, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+    const int* __restrict__ slot, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int Hq, int Hk,
+    int D, int page_size, int write_kv) {
+  const int t = blockIdx.x;
+  bf16_t* row = qkv + (size_t)t * (size_t)(Hq + (write_kv ? 2 * Hk : 0)) * D;
+  const float pos = (float)positions[t];
+  const int s = write_kv ? slot[t] : -1;
+  const int page = s >= 0 ? s / page_size : 0;
+  const int off = s >= 0 ? s - page * page_size : 0;
+  const int half = D >> 1;
+  const int gph = half >> 3;                                  // groups of eight pairs per head
+  const int Hr = Hq + (write_kv ? Hk : 0);
+  for (int idx = threadIdx.x; idx < Hr * gph; idx += blockDim.x) {
+    const int h = idx / gph;
+    const int j0 = (idx - h * gph) * 8;
+    bf16_t* hp = row + (size_t)h * D;
+    const uint4 lo = *reinterpret_cast<const uint4*>(hp + j0);
+    const uint4 hi = *reinterpret_cast<const uint4*>(hp + half + j0);
+    const uint32_t lw[4] = {lo.x, lo.y, lo.z, lo.w}, hw[4] = {hi.x, hi.y, hi.z, hi.w};
+    uint32_t ol[4], oh[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float o0[2], o1[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float a = bf16_bits_to_float(e ? lw[k] >> 16 : lw[k] & 0xffffu);
+        const float b = bf16_bits_to_float(e ? hw[k] >> 16 : hw[k] & 0xffffu);
+        float sn, cs;
+        sincos_reduced(pos * inv_freq[j0 + 2 * k + e], &sn, &cs);
+        o0[e] = a * cs - b * sn;
+        o1[e] = b * cs + a * sn;
+      }
+      ol[k] = (uint32_t)float_to_bf16_bits(o0[0]) | ((uint32_t)float_to_bf16_bits(o0[1]) << 16);
+      oh[k] = (uint32_t)float_to_bf16_bits(o1[0]) | ((uint32_t)float_to_bf16_bits(o1[1]) << 16);
+    }
+    bf16_t* dst = hp;
+    if (h >= Hq) {
+      if (s < 0) continue;
+      dst = k_pages + (((size_t)page * Hk + (h - Hq)) * page_size + off) * D;
+    }
+    *reinterpret_cast<uint4*>(dst + j0) = make_uint4(ol[0], ol[1], ol[2], ol[3]);
+    *reinterpret_cast<uint4*>(dst + half + j0) = make_uint4(oh[0], oh[1], oh[2], oh[3]);
+  }
+  if (s < 0) return;
+  const int gpv = D >> 3;                                     // groups of eight dims per V head
+  for (int idx = threadIdx.x; idx < Hk * gpv; idx += blockDim.x) {
+    const int h = idx / gpv;
+    const int i0 = (idx - h * gpv) * 8;
+    const uint4 v = *reinterpret_cast<const uint4*>(row + (size_t)(Hq + Hk + h) * D + i0);
+    const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+    bf16_t* vp = v_pages + (((size_t)page * Hk + h) * D + i0) * page_size + off;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      vp[(size_t)(2 * k) * page_size].v = (uint16_t)(vw[k] & 0xffffu);
+      vp[(size_t)(2 * k + 1) * page_size].v = (uint16_t)(vw[k] >> 16);
+    }
+  }
+}
+
 extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, const float* inv_freq,
                                 const int* slot, void* k_pages, void* v_pages, int cache_dtype, int T,
                                 int Hq, int Hk, int D, int rot_dim, int adjacent, int page_size,
@@ -250,6 +313,13 @@ extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, 
   if (Hq <= 0 || Hk < 0 || D <= 0 || rot_dim < 0 || rot_dim > D || (rot_dim & 1) || page_size <= 0)
     return SA_ERR_ARG;
   dim3 grid(T), block(256);
+  if (act_dtype == SA_BF16 && cache_dtype == SA_BF16 && !adjacent && rot_dim == D && (D & 15) == 0 &&
+      ((uintptr_t)qkv & 15) == 0) {
+    hipLaunchKernelGGL(rope_kv_write_bf16_vec_kernel, grid, block, 0, stream, (bf16_t*)qkv, positions, inv_freq,
+                       slot, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size, write_kv);
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
 #define GO(TA, TC)                                                                               \
   hipLaunchKernelGGL((rope_kv_write_kernel<TA, TC>), grid, block, 0, stream, (TA*)qkv, positions, \
                      inv_freq, slot, (TC*)k_pages, (TC*)v_pages, Hq, Hk, D, rot_dim, adjacent,   \

@@ -100,7 +100,8 @@ def rope_ref(x, pos, inv_freq, rot, adjacent):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("Hq,Hk,D,rot,adjacent,ps", [(4, 2, 16, 16, False, 4), (3, 1, 48, 32, True, 8),
-                                                     (6, 3, 80, 80, False, 16)])
+                                                     (6, 3, 80, 80, False, 16), (32, 8, 64, 64, False, 16),
+                                                     (5, 5, 112, 112, False, 12)])
 def test_rope_kv_write(dtype, Hq, Hk, D, rot, adjacent, ps):
     from serve_amd import ops
     T, P = 11, 9

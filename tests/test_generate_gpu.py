@@ -377,3 +377,180 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     assert not torch.allclose(wa[-1], wb[-1])
     # the state matters: the last position differs from running the last token alone
     assert not torch.allclose(whole(a[-1:])[0], wa[-1], atol=1e-3)
+
+
+# ---------------------------------------------------------------------------------------------
+# a toy feed-forward with routing and a toy position encoding, defined here, registered, built and
+# stepped beside the framework's own attention
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_other_position_encoding(tmp_path, dtype):
+    """Layers of one model differ: layer 0 has the framework's SwiGLU, layer 1 a feed-forward that
+    sends every token to one of three small experts (router logits in fp32, top 1), and the
+    attention of both layers takes a position encoding from this test that rotates nothing (the
+    order of tokens then enters through the causal mask alone).  Nothing in the framework's files
+    knows these parts.  The oracle is written out below from the plain functions."""
+    from dataclasses import dataclass
+
+    import serve_amd
+    from serve_amd import ops
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.spec import LayerSpec, ModelSpec, PartSpec, RunEntry
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    from serve_amd.parts.base import ParamRequest, Part
+    from serve_amd.parts.linear import linear
+    from serve_amd.weights.loader import write_random_model
+    from tests.plain import llama_plain as P
+
+    d, Hq, Hk, D, I, E, V, L = 48, 3, 1, 16, 40, 3, 61, 2
+
+    class NoRotation(Part):
+        """Position encoding that leaves q and k as they are; it still has to put k and v into
+        the cache, which is the position part's job in the framework's attention."""
+
+        def __init__(self, head_dim):
+            self.head_dim = head_dim
+
+        def load(self, tensors, rt):
+            self.none = torch.empty(0, dtype=torch.float32, device=rt.device)
+
+        def rotate_and_store(self, qkv, positions, slots, cache, num_heads, num_kv_heads):
+            ops.rope_kv_write(qkv, positions, self.none, slots,
+                              None if slots is None else cache.k_pages, None if slots is None else cache.v_pages,
+                              num_heads, num_kv_heads, self.head_dim, 0, False,
+                              0 if cache is None else cache.page_size)
+
+    class TopOneExperts(Part):
+        def __init__(self, hidden_size, intermediate_size, num_experts):
+            self.d, self.i, self.e = hidden_size, intermediate_size, num_experts
+
+        def param_requests(self):
+            reqs = [ParamRequest("router.weight", (self.e, self.d))]
+            for e in range(self.e):
+                reqs += [ParamRequest(f"experts.{e}.gate.weight", (self.i, self.d)),
+                         ParamRequest(f"experts.{e}.up.weight", (self.i, self.d)),
+                         ParamRequest(f"experts.{e}.down.weight", (self.d, self.i))]
+            return reqs
+
+        def load(self, tensors, rt):
+            self.rt, self.w = rt, tensors
+
+        def forward(self, h, ctx):
+            logits = linear(h.float().contiguous(), self.w["router.weight"].float().contiguous())   # fp32
+            choice = torch.argmax(logits, dim=-1)
+            out = torch.zeros((h.shape[0], self.d), dtype=torch.float32, device=h.device)
+            for e in range(self.e):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel() == 0:
+                    continue
+                x = h[rows].contiguous()
+                gu = torch.cat([linear(x, self.w[f"experts.{e}.gate.weight"]),
+                                linear(x, self.w[f"experts.{e}.up.weight"])], dim=1).contiguous()
+                a = torch.empty((x.shape[0], self.i), dtype=h.dtype, device=h.device)
+                ops.silu_mul(gu, a)
+                out[rows] = linear(a, self.w[f"experts.{e}.down.weight"], out_dtype=torch.float32)
+            return out
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture = "ToyRoutedLM"
+
+        def to_hf_dict(self):
+            return {"architectures": [self.architecture]}
+
+        @staticmethod
+        def from_hf_dict(_):
+            return ToyConfig()
+
+    def build(cfg):
+        norm = PartSpec("rmsnorm", {"size": d, "eps": 1e-5})
+        attn = PartSpec("gqa_attention", {"hidden_size": d, "num_heads": Hq, "num_kv_heads": Hk, "head_dim": D,
+                                          "scale": D ** -0.5,
+                                          "position": PartSpec("no_rotation", {"head_dim": D})})
+        layers = []
+        for i in range(L):
+            p = f"toy.{i}."
+            weights = {"mixer.q_proj.weight": p + "q", "mixer.k_proj.weight": p + "k", "mixer.v_proj.weight": p + "v",
+                       "mixer.o_proj.weight": p + "o", "mixer_norm.weight": p + "n1", "ffn_norm.weight": p + "n2"}
+            if i == 0:
+                ffn = PartSpec("swiglu", {"hidden_size": d, "intermediate_size": I})
+                weights.update({"ffn.gate_proj.weight": p + "gate", "ffn.up_proj.weight": p + "up",
+                                "ffn.down_proj.weight": p + "down"})
+            else:
+                ffn = PartSpec("top_one_experts", {"hidden_size": d, "intermediate_size": I, "num_experts": E})
+                weights["ffn.router.weight"] = p + "router"
+                for e in range(E):
+                    for n in ("gate", "up", "down"):
+                        weights[f"ffn.experts.{e}.{n}.weight"] = p + f"e{e}.{n}"
+            layers.append(LayerSpec(mixer=attn, ffn=ffn, mixer_norm=norm, ffn_norm=norm, weights=weights))
+        return ModelSpec(architecture=cfg.architecture, vocab_size=V, hidden_size=d,
+                         embedding=PartSpec("token_embedding", {"vocab_size": V, "hidden_size": d}),
+                         layers=layers, run_order=[RunEntry(i, i) for i in range(L)], final_norm=norm,
+                         lm_head=PartSpec("linear_head", {"vocab_size": V, "hidden_size": d, "tied": True}),
+                         weights={"embedding.weight": "toy.embed", "final_norm.weight": "toy.norm",
+                                  "lm_head.weight": "toy.head"})
+
+    serve_amd.register_part("position", "no_rotation", NoRotation)
+    serve_amd.register_part("feed_forward", "top_one_experts", TopOneExperts)
+    serve_amd.register_architecture("ToyRoutedLM", ToyConfig.from_hf_dict, build)
+    folder = write_random_model(str(tmp_path / "toy"), ToyConfig(), seed=11)
+    eng = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=4, num_pages=24, max_context=64,
+                                                 max_requests=3))
+    assert not eng.model.graph_safe()                     # the routed part reads back to the host
+    rng = random.Random(6)
+    a, b = util.random_tokens(rng, 21, V), util.random_tokens(rng, 9, V)
+
+    # the oracle, whole sequences, fp64
+    w = {k: t.double() for k, t in util.plain_weights(folder).items()}
+
+    def oracle(tokens):
+        x = w["toy.embed"][torch.tensor(tokens)]
+        margins = []
+        for i in range(L):
+            p = f"toy.{i}."
+            h = P.rms_norm(x, w[p + "n1"], 1e-5)
+            S = h.shape[0]
+            q, k, v = (h @ w[p + "q"].T).view(S, Hq, D), (h @ w[p + "k"].T).view(S, Hk, D), (h @ w[p + "v"].T).view(S, Hk, D)
+            x = x + P.causal_attention(q, k, v).reshape(S, Hq * D) @ w[p + "o"].T
+            h = P.rms_norm(x, w[p + "n2"], 1e-5)
+            if i == 0:
+                x = x + P.swiglu(h, w[p + "gate"], w[p + "up"], w[p + "down"])
+            else:
+                logits = h @ w[p + "router"].T
+                top = torch.topk(logits, 2, dim=-1).values
+                margins.append((top[:, 0] - top[:, 1]).min().item())
+                choice = torch.argmax(logits, -1)
+                y = torch.zeros_like(x)
+                for e in range(E):
+                    m = choice == e
+                    y[m] = P.swiglu(h[m], w[p + f"e{e}.gate"], w[p + f"e{e}.up"], w[p + f"e{e}.down"])
+                x = x + y
+        return P.rms_norm(x, w["toy.norm"], 1e-5) @ w["toy.embed"].T, min(margins)
+
+    wa, ma = oracle(a)
+    wb, mb = oracle(b)
+    eng.runner.admit("a")
+    eng.runner.admit("b")
+    r1 = eng.step([Segment("a", a[:13], list(range(13))), Segment("b", b[:2], [0, 1])])
+    r2 = eng.step([Segment("b", b[2:], list(range(7))), Segment("a", a[13:14], [0])])
+    r3 = eng.step([Segment("a", a[14:], list(range(7)))])
+    got_a = torch.cat([r1[:13], r2[7:], r3]).double().cpu()
+    got_b = torch.cat([r1[13:], r2[:7]]).double().cpu()
+    if dtype == "float32":
+        assert min(ma, mb) > 1e-4, "a router decision of the oracle is too close to call in fp32: change the seed"
+        util.assert_close(got_a, wa, dtype, "toy routed a")
+        util.assert_close(got_b, wb, dtype, "toy routed b")
+    else:
+        # bf16 may route a token with a near tie elsewhere; rows whose decision is clear must agree
+        tol = util.TOL[dtype]
+        close = ((got_a - wa).abs() <= tol["atol"] + tol["rtol"] * wa.abs()).all(dim=-1).float().mean().item()
+        assert close >= 0.8, f"only {close:.2f} of the rows agree with the oracle in bf16"
+    # the order of tokens matters although nothing is rotated: swap two prompt tokens
+    swapped = list(a)
+    swapped[1], swapped[2] = swapped[2], swapped[1]
+    eng.runner.release("a")
+    eng.runner.release("b")
+    eng.runner.admit("s")
+    rs = eng.step([Segment("s", swapped, [len(swapped) - 1])])
+    assert not torch.allclose(rs[0].double().cpu(), got_a[-1], atol=1e-3)

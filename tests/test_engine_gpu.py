@@ -167,3 +167,47 @@ def test_far_key_stands_out(tmp_path, dtype):
     tokens = util.random_tokens(rng, 400, util.TINY[name][0].vocab_size)
     got = run_portions(engine, "r", tokens, [3, 61, 130, 2, 97, 7, 99, 1])
     util.assert_close(got, util.plain_logits(folder, tokens), dtype, "far keys")
+
+
+# ---------------------------------------------------------------------------------------------
+# sizes that no kernel likes: the engine takes them (through its general kernels) or refuses them,
+# never a wrong result
+# ---------------------------------------------------------------------------------------------
+ODD = {
+    # width, feed-forward and head size no multiples of 8 or 16, as many KV heads as heads
+    "odd1": dict(vocab_size=333, hidden_size=100, intermediate_size=100, num_hidden_layers=2,
+                 num_attention_heads=5, num_key_value_heads=5, head_dim=20, rms_norm_eps=1e-5,
+                 rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False),
+    # head size 48 (a multiple of 16 that is none of 32), group of 2, scaled rotation
+    "odd2": dict(vocab_size=70, hidden_size=72, intermediate_size=136, num_hidden_layers=1,
+                 num_attention_heads=6, num_key_value_heads=3, head_dim=48, rms_norm_eps=1e-6,
+                 rope_theta=500000.0, rope_scaling=dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                                        original_max_position_embeddings=32),
+                 tie_word_embeddings=True),
+    # head size 128, one KV head, a prime vocabulary
+    "odd3": dict(vocab_size=4099, hidden_size=256, intermediate_size=520, num_hidden_layers=2,
+                 num_attention_heads=2, num_key_value_heads=1, head_dim=128, rms_norm_eps=1e-5,
+                 rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True),
+}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [12, 32])
+@pytest.mark.parametrize("name", sorted(ODD))
+def test_odd_sizes(tmp_path, name, page_size, dtype):
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.llama import Llama3RopeScaling, LlamaConfig
+    from serve_amd.engine.engine import Engine
+    from serve_amd.weights.loader import write_random_model
+    kw = dict(ODD[name])
+    if kw["rope_scaling"]:
+        kw["rope_scaling"] = Llama3RopeScaling(**kw["rope_scaling"])
+    cfg = LlamaConfig(**kw)
+    folder = write_random_model(str(tmp_path / name), cfg, seed=5)
+    engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=page_size, num_pages=16,
+                                                    max_context=16 * page_size, max_requests=4,
+                                                    max_tokens_per_step=4096, prefill_chunk=4096))
+    rng = random.Random(1)
+    tokens = util.random_tokens(rng, 90, cfg.vocab_size)
+    got = run_portions(engine, "r", tokens, [70, 2, 17, 1])
+    util.assert_close(got, util.plain_logits(folder, tokens), dtype, f"{name} page {page_size}")

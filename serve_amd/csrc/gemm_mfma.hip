@@ -523,16 +523,16 @@ static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, 
       if (four) GO(1, 4, 2, 4);
       GO(1, 2, 2, 4);
     }
-    if (four) GO(2, 4, 4, 2);        // many: 128 a workgroup, which halves the activation traffic
-    GO(2, 2, 4, 2);
+    if (four) GO(1, 4, 8, 2);        // many: 128 a workgroup, which halves the activation traffic
+    GO(1, 2, 8, 2);
   }
   if constexpr (EPI == EPI_QKV_ROPE) {  // few rows again: one tile a workgroup, K cut eight ways
     if (four) GO(1, 4, 1, 8);
     GO(1, 2, 1, 8);
   }
   if constexpr (EPI == EPI_SWIGLU) {
-    if (four) GO(2, 4, 2, 4);
-    GO(2, 2, 2, 4);
+    if (four) GO(2, 4, 2, 2);
+    GO(2, 2, 2, 2);
   }
 #undef GO
   return SA_ERR_ARG;

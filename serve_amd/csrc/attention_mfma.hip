@@ -333,11 +333,32 @@ __device__ __forceinline__ void attention_tile(
         acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
   };
 
-  // Three buffers in turn: the loads of the next two blocks are in flight while one is computed.
+  // Three buffers in turn: the loads of the next two blocks are in flight while one is computed
+  // (two buffers, one block in flight, for prompt tiles of head sizes above 64, whose blocks are
+  // twice as large and would push the registers over the edge).
   // The loads carry no conditions: a block beyond the last is read from clamped keys and pages and
   // never used.  With a branch around them the compiler no longer knows how many loads are in
   // flight where a block's data is awaited, and waits for all of them, the newest included.
-  if (b0 < b1) {
+  if (b0 < b1 && HD > 64 && NT > 1) {
+    Block buf_a, buf_b;
+    prefetch_pages(b0);
+    load_block(b0, buf_a);
+    int kb = b0;
+    for (; kb + 2 <= b1; kb += 2) {
+      if (kb >= full_lo && kb + 1 <= full_hi) {
+        load_block(kb + 1, buf_b);
+        compute(kb, buf_a, Unmasked{});
+        load_block(kb + 2, buf_a);
+        compute(kb + 1, buf_b, Unmasked{});
+      } else {
+        load_block(kb + 1, buf_b);
+        compute(kb, buf_a, Masked{});
+        load_block(kb + 2, buf_a);
+        compute(kb + 1, buf_b, Masked{});
+      }
+    }
+    if (kb < b1) compute(kb, buf_a, Masked{});
+  } else if (b0 < b1) {
     Block buf_a, buf_b, buf_c;
     prefetch_pages(b0);
     load_block(b0, buf_a);

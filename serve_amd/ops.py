@@ -378,9 +378,12 @@ def attention_splits(decode_only: bool, num_segments: int, num_kv_heads: int, ma
 def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                          v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                          ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int, scale: float,
-                         window: Optional[int], num_splits: int = 1) -> torch.Tensor:
+                         window: Optional[int], num_splits: int = 1, seg_begin: int = 0,
+                         seg_count: Optional[int] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores (head sizes 16..128 in steps of 16, page sizes that are
-    multiples of 4)."""
+    multiples of 4).  `seg_begin`, `seg_count`: run only these segments of the step (their
+    tokens' rows of `out` are written, the others left alone); `num_tokens` then is the number of
+    tokens up to the end of the last of them."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
     P, Hk, page_size, D = k_pages.shape
     _check(mfma_attention_available(q, k_pages, q_row_stride),
@@ -390,15 +393,26 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
            "v_pages must be bf16 [P, Hk, D, page_size]")
     _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
     T = num_tokens
-    _check(out.shape == (T, num_heads * D) and out.dtype == torch.bfloat16, "attention output must be bf16 [T, Hq D]")
+    _check(out.dim() == 2 and out.shape[0] >= T and out.shape[1] == num_heads * D and out.dtype == torch.bfloat16,
+           "attention output must be bf16 [T, Hq D]")
     _check(q.numel() >= (T - 1) * q_row_stride + num_heads * D if T else True, "q is too short")
     _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
-    B = block_table.shape[0]
-    _i32(cu_q, B + 1, "cu_q")
-    _i32(ctx_len, B, "ctx_len")
+    B_all = block_table.shape[0]
+    _i32(cu_q, B_all + 1, "cu_q")
+    _i32(ctx_len, B_all, "ctx_len")
+    B = B_all - seg_begin if seg_count is None else seg_count
+    _check(0 <= seg_begin and B >= 0 and seg_begin + B <= B_all, "segment range out of bounds")
+    if B == 0:
+        return out
+    if seg_begin or B != B_all:
+        block_table = block_table[seg_begin: seg_begin + B]
+        cu_q = cu_q[seg_begin: seg_begin + B + 1]
+        ctx_len = ctx_len[seg_begin: seg_begin + B]
     _check(1 <= max_q_len <= max(T, 1) and num_splits >= 1, "max_q_len / num_splits out of range")
     part_o = part_ml = None
     if num_splits > 1:
+        # the parts are indexed by token, and the merge runs over tokens 0 .. T-1
+        _check(seg_begin == 0, "a split key range needs the segments to start at token 0")
         part_o = torch.empty((T * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
     lib = load_library("attention_mfma", {"HEAD_DIM": D})
@@ -414,6 +428,30 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
 # dispatch between kernels of the same operation
 # ---------------------------------------------------------------------------------------------
 
+def _attention_launches(ctx):
+    """How a step's segments go to the matrix-core attention kernel.  Single decoded tokens take
+    16-row tiles and a split key range, prompt portions larger tiles: a step that begins with
+    decoding requests and goes on with prompt portions (the order the scheduler gives) is run as
+    two launches, each with the tiles that suit it.  Computed once per step and kept on `ctx`."""
+    plan = getattr(ctx, "_attention_launches", None)
+    if plan is not None:
+        return plan
+    B, T = ctx.num_segments, ctx.num_tokens
+    if ctx.decode_only or not ctx.q_lens:
+        plan = [(0, B, T, ctx.max_q_len, ctx.max_ctx_len)]
+    else:
+        nd = 0
+        while nd < B and ctx.q_lens[nd] == 1:
+            nd += 1
+        if nd < 4 or nd == B:
+            plan = [(0, B, T, ctx.max_q_len, ctx.max_ctx_len)]
+        else:
+            plan = [(0, nd, nd, 1, max(ctx.ctx_lens[:nd])),
+                    (nd, B - nd, T, max(ctx.q_lens[nd:]), max(ctx.ctx_lens[nd:]))]
+    ctx._attention_launches = plan
+    return plan
+
+
 def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                     v_pages: torch.Tensor, block_table: torch.Tensor, ctx, num_heads: int, scale: float,
                     window: Optional[int]) -> torch.Tensor:
@@ -421,8 +459,12 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
     (`serve_amd.engine.batch.StepContext`): the matrix-core kernel for bf16 where it takes the
     sizes, else the general fp32-arithmetic kernel."""
     if mfma_attention_available(q, k_pages, q_row_stride):
-        splits = attention_splits(ctx.decode_only, ctx.num_segments, k_pages.shape[1], ctx.max_ctx_len)
-        return paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
-                                    ctx.num_tokens, ctx.max_q_len, num_heads, scale, window, splits)
+        Hk = k_pages.shape[1]
+        # (first segment, segments, tokens up to their end, longest portion, longest context)
+        for s0, n, t_end, max_q, max_ctx in _attention_launches(ctx):
+            splits = attention_splits(max_q == 1, n, Hk, max_ctx)
+            paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
+                                 t_end, max_q, num_heads, scale, window, splits, s0, n)
+        return out
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                   ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

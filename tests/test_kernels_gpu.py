@@ -189,6 +189,16 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     if kernel == "simple":
         ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
                                    T, Hq, scale, window)
+    elif kernel == "dispatch":
+        # the way the attention part calls it: the step's facts decide how many launches there are
+        from types import SimpleNamespace
+        q_lens, ctx_lens = [ql for _, ql in segs], [c + ql for c, ql in segs]
+        ctx = SimpleNamespace(num_segments=B, num_tokens=T, cu_q=cu_q, ctx_len=ctx_len, seg_of_token=seg_of_token,
+                              q_lens=q_lens, ctx_lens=ctx_lens, max_q_len=max(q_lens), max_ctx_len=max(ctx_lens),
+                              decode_only=all(n == 1 for n in q_lens))
+        out.fill_(float("nan"))
+        ops.paged_attention(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), ctx, Hq, scale, window)
+        assert len(ctx._attention_launches) == splits          # here: the number of launches expected
     else:
         ops.paged_attention_mfma(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
                                  max(ql for _, ql in segs), Hq, scale, window, splits)
@@ -315,6 +325,18 @@ def test_paged_attention_mfma_mixed(Hq, Hk, D, ps):
 def test_paged_attention_mfma_decode_with_splits(Hq, Hk, D, ps, splits):
     segs = [(12, 1), (0, 1), (130, 1), (517, 1), (31, 1), (32, 1), (63, 1), (64, 1)]
     attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=300 + D, kernel="mfma", splits=splits)
+
+
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(8, 2, 64, 16), (6, 2, 128, 16), (3, 1, 32, 8), (4, 4, 48, 12)])
+def test_paged_attention_step_of_decodes_then_prompt_portions(Hq, Hk, D, ps):
+    """A step that begins with decoding requests and goes on with prompt portions runs as two
+    launches (16-row tiles and split keys for the former); any other order runs as one."""
+    decodes = [(12, 1), (0, 1), (130, 1), (700, 1), (31, 1), (32, 1), (63, 1), (64, 1), (5, 1)]
+    prompts = [(0, 7), (63, 5), (5, 70), (31, 2), (0, 33)]
+    attention_case("bfloat16", Hq, Hk, D, ps, decodes + prompts, seed=400 + D, kernel="dispatch", splits=2)
+    attention_case("bfloat16", Hq, Hk, D, ps, decodes[:3] + prompts, seed=401 + D, kernel="dispatch", splits=1)
+    attention_case("bfloat16", Hq, Hk, D, ps, prompts + decodes, seed=402 + D, kernel="dispatch", splits=1)
+    attention_case("bfloat16", Hq, Hk, D, ps, decodes, seed=403 + D, kernel="dispatch", splits=1)
 
 
 def test_paged_attention_mfma_window_standout_and_long_prompt():

@@ -120,9 +120,14 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
             raise ValueError(f"request {s.req_id!r} brings no tokens")
         if s.req_id not in cache:
             raise KeyError(f"request {s.req_id!r} is not admitted")
-        for t in s.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise ValueError(f"token id {t} of request {s.req_id!r} is outside the vocabulary [0, {vocab_size})")
+        if len(s.tokens) == 1:
+            lo = hi = int(s.tokens[0])
+        else:
+            arr = np.asarray(s.tokens)
+            lo, hi = int(arr.min()), int(arr.max())
+        if lo < 0 or hi >= vocab_size:
+            bad = lo if lo < 0 else hi
+            raise ValueError(f"token id {bad} of request {s.req_id!r} is outside the vocabulary [0, {vocab_size})")
         for w in s.want:
             if not 0 <= int(w) < len(s.tokens):
                 raise ValueError(f"request {s.req_id!r} wants the logits at place {w} of {len(s.tokens)} tokens")
@@ -177,28 +182,44 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         facts = dict(q_lens=[1] * B, ctx_lens=ctx_lens, max_q_len=1, max_ctx_len=max(ctx_lens),
                      max_pages=MP, decode_only=True)
         return lay, host, facts
-    cu = 0
-    r_i = 0
-    q_lens, ctx_lens = [], []
-    for i, (s, b, a) in enumerate(zip(segments, before, after)):
-        n = len(s.tokens)
-        host[lay.token_ids + cu: lay.token_ids + cu + n] = np.asarray(s.tokens, dtype=np.int32)
-        host[lay.positions + cu: lay.positions + cu + n] = np.arange(b, a, dtype=np.int32)
-        host[lay.seg_of_token + cu: lay.seg_of_token + cu + n] = i
-        host[lay.cu_q + i] = cu
-        host[lay.ctx_len + i] = a
-        host[lay.state_slots + i] = cache.slot_of(s.req_id)
-        for w in s.want:
-            host[lay.logit_rows + r_i] = cu + int(w)
-            r_i += 1
+    # per segment, without a loop: token offsets, context lengths, state slots, block tables
+    n = B_real
+    q_lens = [len(s.tokens) for s in segments]
+    ctx_lens = list(after)
+    cu_np = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(q_lens, out=cu_np[1:])
+    before_np = np.asarray(before, dtype=np.int64)
+    slots_np = np.fromiter((cache.slot_of(s.req_id) for s in segments), dtype=np.int64, count=n)
+    host[lay.cu_q: lay.cu_q + n] = cu_np[:n]
+    host[lay.ctx_len: lay.ctx_len + n] = after
+    host[lay.state_slots: lay.state_slots + n] = slots_np
+    host[lay.logit_rows: lay.logit_rows + R] = [int(c) + int(w) for s, c in zip(segments, cu_np) for w in s.want]
+    rows_of = []
+    for g in range(G):
+        rows = cache.table_rows[g][slots_np]
+        rows_of.append(rows)
+        host[lay.block_tables[g]: lay.block_tables[g] + n * MP].reshape(n, MP)[:] = rows[:, :MP]
+    # per token: the single-token segments together, the others one by one
+    q_np = np.asarray(q_lens)
+    one = np.nonzero(q_np == 1)[0]
+    if one.size:
+        at = cu_np[one]
+        b1 = before_np[one]
+        host[lay.token_ids + at] = [segments[i].tokens[0] for i in one]
+        host[lay.positions + at] = b1
+        host[lay.seg_of_token + at] = one
         for g in range(G):
-            table = np.asarray(cache.block_table(s.req_id, g), dtype=np.int32)
-            host[lay.block_tables[g] + i * MP: lay.block_tables[g] + i * MP + len(table)] = table
-            pos = np.arange(b, a)
-            host[lay.slots[g] + cu: lay.slots[g] + cu + n] = table[pos // ps] * ps + pos % ps
-        cu += n
-        q_lens.append(n)
-        ctx_lens.append(a)
+            host[lay.slots[g] + at] = rows_of[g][one, b1 // ps] * ps + b1 % ps
+    for i in np.nonzero(q_np != 1)[0]:
+        s, b, a, c0 = segments[i], before[i], after[i], int(cu_np[i])
+        m = a - b
+        host[lay.token_ids + c0: lay.token_ids + c0 + m] = np.asarray(s.tokens, dtype=np.int32)
+        host[lay.positions + c0: lay.positions + c0 + m] = np.arange(b, a, dtype=np.int32)
+        host[lay.seg_of_token + c0: lay.seg_of_token + c0 + m] = i
+        pos = np.arange(b, a)
+        for g in range(G):
+            host[lay.slots[g] + c0: lay.slots[g] + c0 + m] = rows_of[g][i, pos // ps] * ps + pos % ps
+    cu = int(cu_np[n])
     for j in range(pad):           # inert segments: one token, one visible key, nothing stored
         i = B_real + j
         host[lay.seg_of_token + cu] = i

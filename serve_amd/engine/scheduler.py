@@ -29,7 +29,7 @@ from ..config.engine import EngineConfig
 from .batch import Segment
 
 
-@dataclass
+@dataclass(eq=False)                     # requests are told apart by identity, not by their fields
 class GenerationRequest:
     req_id: int
     prompt: List[int]
@@ -292,9 +292,9 @@ class Scheduler:
         if any(n != 1 or not s or r.keep_logits for r, n, s in zip(plan.requests, plan.counts, plan.samples)):
             return False
         if self._inflight is not None:
-            before = self._inflight[1]
+            before = {id(r) for r in self._inflight[1]}
             for r in plan.requests:
-                if r.generated and r.generated[-1] is None and r not in before:
+                if r.generated and r.generated[-1] is None and id(r) not in before:
                     return False
         return True
 

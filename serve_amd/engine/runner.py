@@ -101,9 +101,13 @@ class ModelRunner:
         self.storage = CacheStorage(rt, creq, sreq, self.windows, num_pages, cfg.page_size, cfg.max_requests)
         self._graphs = {}
         # tokens sampled by the latest decode launch, by row: the next launch may read them here
-        self.sampled = torch.zeros(GRAPH_BATCHES[-1], dtype=torch.int32, device=rt.device)
+        self.sampled = torch.zeros(max(GRAPH_BATCHES[-1], cfg.max_requests), dtype=torch.int32, device=rt.device)
         self._row_of = {}
         self._use_graphs = bool(cfg.use_graphs) and model.graph_safe()
+        # steps launched ahead of the host need parts that never read back from the device
+        self._launch_ahead = model.graph_safe()
+        self._host_tokens = None            # pinned ring for the tokens of steps launched eagerly
+        self._eager_launches = 0
 
     # -- requests -------------------------------------------------------------------------------
     def admit(self, req_id) -> bool:
@@ -220,6 +224,9 @@ class ModelRunner:
     def can_decode_async(self, n: int) -> bool:
         return self._use_graphs and 0 < n <= GRAPH_BATCHES[-1]
 
+    def can_launch_ahead(self) -> bool:
+        return self._launch_ahead
+
     @torch.inference_mode()
     def decode_launch(self, req_ids: Sequence, tokens: Sequence[Optional[int]], temperatures: Sequence[float],
                       keys: Sequence[int]) -> DecodeHandle:
@@ -242,3 +249,54 @@ class ModelRunner:
         for r, n in zip(req_ids, ctx_lens):
             self.cache.trim(r, n)
         return DecodeHandle(host, ev, len(req_ids))
+
+    @torch.inference_mode()
+    def step_launch(self, req_ids: Sequence, tokens: Sequence[Sequence[Optional[int]]], samples: Sequence[bool],
+                    temperatures: Sequence[float], keys: Sequence[int]) -> DecodeHandle:
+        """Launch any step (prompt portions beside single tokens) with sampling on the device, and
+        return at once: the eager counterpart of `decode_launch`.  tokens[i] are request i's next
+        tokens; a single token may be None for "the token that the previous launch sampled for
+        this request".  samples[i]: whether a token is drawn from the logits at request i's last
+        place; `temperatures` and `keys` belong to those requests, in order, and so do the tokens
+        of the handle."""
+        with torch.cuda.device(self.rt.device):
+            segments = [Segment(r, [0 if t is None else t for t in toks], [len(toks) - 1] if smp else [])
+                        for r, toks, smp in zip(req_ids, tokens, samples)]
+            lay, host, facts = plan_step(segments, self.cache, self.vocab_size)
+            T, R = lay.T, lay.R
+            # behind the step's own arrays: where each token comes from, and the sampling inputs
+            off_src = lay.total
+            off_temps = off_src + _pad4(T)
+            off_keys = off_temps + _pad4(R)
+            buf = np.zeros(off_keys + _pad4(2 * R), dtype=np.int32)
+            buf[: lay.total] = host
+            src = buf[off_src: off_src + T]
+            src[:] = -1
+            cu = host[lay.cu_q: lay.cu_q + len(segments)]
+            for i, (r, toks) in enumerate(zip(req_ids, tokens)):
+                if toks[0] is None:
+                    if len(toks) != 1:
+                        raise ValueError("only a single token can be left to the device")
+                    src[cu[i]] = self._row_of[r]
+            buf[off_temps: off_temps + R].view(np.float32)[:] = np.asarray(temperatures, dtype=np.float32)
+            buf[off_keys: off_keys + 2 * R].view(np.int64)[:] = np.asarray(keys, dtype=np.int64)
+            dev = torch.from_numpy(buf).to(self.rt.device)
+            ctx = context_from(lay, dev, facts)
+            ctx.src_row = dev[off_src: off_src + T]
+            ctx.prev_tokens = self.sampled
+            logits = self.model.forward(ctx, self.storage.layers)
+            if R:
+                ops.sample(logits, dev[off_temps: off_temps + R].view(torch.float32),
+                           dev[off_keys: off_keys + 2 * R].view(torch.int64), self.sampled[:R])
+            self._row_of = {r: i for i, r in enumerate(r for r, smp in zip(req_ids, samples) if smp)}
+            if self._host_tokens is None:
+                self._host_tokens = [torch.zeros(self.sampled.numel(), dtype=torch.int32).pin_memory() for _ in range(2)]
+            host_tokens = self._host_tokens[self._eager_launches & 1]
+            self._eager_launches += 1
+            host_tokens[:R].copy_(self.sampled[:R], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+        for r, n in zip(req_ids, facts["ctx_lens"]):
+            self.cache.trim(r, n)
+        return DecodeHandle(host_tokens, ev, R)
+

@@ -258,8 +258,12 @@ class Scheduler:
         if not plan.requests:
             self._resolve()
             return False
-        if self._pipelinable(plan):
+        ahead = self._pipelinable(plan)
+        if ahead == "decode":
             self._launch_decode(plan)
+            return True
+        if ahead == "any":
+            self._launch_step(plan)
             return True
         self._resolve()                       # the tokens of the step in flight are needed on the host
         segments = []
@@ -283,20 +287,50 @@ class Scheduler:
         return True
 
     # -- decode steps with the host one step ahead ---------------------------------------------------
-    def _pipelinable(self, plan: StepPlan) -> bool:
-        """A step of single tokens that all sample, whose finishing does not depend on the tokens
-        (no stop tokens) and whose logits nobody keeps: it can be launched before the tokens of
-        the step before it have reached the host, which then are fed back on the device."""
-        if not self.async_decode or not self.runner.can_decode_async(len(plan.requests)):
-            return False
-        if any(n != 1 or not s or r.keep_logits for r, n, s in zip(plan.requests, plan.counts, plan.samples)):
-            return False
+    def _pipelinable(self, plan: StepPlan) -> Optional[str]:
+        """Whether the step can be launched before the tokens of the step before it have reached
+        the host, which then are fed back on the device: its finishing must not depend on the
+        tokens (no stop tokens), nobody keeps its logits, and a request whose last token is still
+        on the device must have got it from the step in flight.  "decode": single tokens that all
+        sample, replayed from a graph; "any": prompt portions too, launched kernel by kernel;
+        None: the host needs the tokens first."""
+        if not self.async_decode:
+            return None
+        if any(r.keep_logits for r in plan.requests):
+            return None
         if self._inflight is not None:
             before = {id(r) for r in self._inflight[1]}
             for r in plan.requests:
                 if r.generated and r.generated[-1] is None and id(r) not in before:
-                    return False
-        return True
+                    return None
+        if (self.runner.can_decode_async(len(plan.requests))
+                and all(n == 1 and s for n, s in zip(plan.counts, plan.samples))):
+            return "decode"
+        if getattr(self.runner, "can_launch_ahead", lambda: False)():
+            return "any"
+        return None
+
+    def _launch_step(self, plan: StepPlan) -> None:
+        """A step with prompt portions, launched ahead of the host like `_launch_decode`."""
+        from ..sampling.sampler import _signed, row_key
+        reqs = plan.requests
+        tokens = [r.tokens_between(r.fed, r.fed + n) for r, n in zip(reqs, plan.counts)]
+        samplers = [r for r, s in zip(reqs, plan.samples) if s]
+        keys = [_signed(row_key(self.sampler.seed, r.req_id, len(r.generated))) for r in samplers]
+        handle = self.runner.step_launch([r.req_id for r in reqs], tokens, plan.samples,
+                                         [r.temperature for r in samplers], keys)
+        previous, self._inflight = self._inflight, (handle, samplers, [len(r.generated) for r in samplers])
+        self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in reqs], counts=list(plan.counts),
+                                  sampled=[r.req_id for r in samplers]))
+        self.steps += 1
+        for r, n in zip(reqs, plan.counts):
+            r.fed += n
+        for r in samplers:
+            r.generated.append(None)          # filled in when the step's tokens are read back
+            if r.done():
+                self._finish(r)
+        if previous is not None:
+            self._read_back(previous)
 
     def _launch_decode(self, plan: StepPlan) -> None:
         from ..sampling.sampler import _signed, row_key

@@ -290,13 +290,16 @@ def split_k_parts(M: int, N: int, K: int) -> int:
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """bf16 product: the weight-streaming kernel for few rows, the BLAS library for many (the
-    reference leaves all of its products to the library, serve/model.py:80-82,95,97,159).  The
-    library writes bf16; fp32 output always takes the kernel."""
-    if a.shape[0] <= SKINNY_MAX_ROWS or out.dtype != torch.bfloat16:
+    """bf16 product: the weight-streaming kernels for few rows, the BLAS library for many (the
+    reference leaves all of its products to the library, serve/model.py:80-82,95,97,159); both
+    write bf16 or fp32."""
+    if a.shape[0] <= SKINNY_MAX_ROWS:
         return gemm_bf16_skinny(a, w, out)
     _dev(a, w, out)
-    torch.mm(a, w.t(), out=out)
+    if out.dtype == torch.bfloat16:
+        torch.mm(a, w.t(), out=out)
+    else:
+        torch.mm(a, w.t(), out_dtype=out.dtype, out=out)
     return out
 
 

@@ -28,12 +28,14 @@ HBM_PEAK = 8.0e12            # bytes/s, MI355X
 BF16_PEAK = 2.5e15           # dense bf16 MFMA flop/s, MI355X
 
 
-def model_config(layers: int):
-    from serve_amd.config.llama import Llama3RopeScaling, LlamaConfig
-    return LlamaConfig(vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_hidden_layers=layers,
-                       num_attention_heads=32, num_key_value_heads=8, head_dim=64, rms_norm_eps=1e-5,
-                       rope_theta=500000.0,
-                       rope_scaling=Llama3RopeScaling(32.0, 1.0, 4.0, 8192), tie_word_embeddings=True)
+def model_config(layers: int, shape: str = "llama-1b"):
+    """The default is the Llama-3.2-1B shape; `shape` names another one of serve_amd.benchmark.SHAPES
+    (for measurements beside the headline one)."""
+    from dataclasses import replace
+
+    from serve_amd.benchmark import SHAPES
+    cfg = SHAPES[shape]
+    return replace(cfg, num_hidden_layers=layers if layers > 0 else cfg.num_hidden_layers)
 
 
 def weight_bytes(cfg) -> int:
@@ -116,7 +118,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--layers", type=int, default=16, help="fewer than 16 only to save time; both are reported")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has, only to save time; "
+                    "both numbers are reported (0: all)")
+    ap.add_argument("--shape", default="llama-1b", help="llama-1b (the headline measurement), llama-3b, llama-8b")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch-1/64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own short JSON line")
@@ -129,8 +133,9 @@ def main() -> int:
     from serve_amd.config.engine import EngineConfig
     from serve_amd.engine.engine import Engine
 
-    full_layers = 16
-    cfg = model_config(args.layers)
+    cfg = model_config(args.layers, args.shape)
+    full_layers = model_config(0, args.shape).num_hidden_layers
+    shape_name = {"llama-1b": "Llama-3.2-1B", "llama-3b": "Llama-3.2-3B", "llama-8b": "Llama-3.1-8B"}.get(args.shape, args.shape)
     page = 16
     pages_needed = args.batch * (-(-args.context // page)) + 64 * (-(-600 // page)) + 256
     ecfg = EngineConfig(dtype="bfloat16", page_size=page, num_pages=pages_needed, max_context=args.context,
@@ -155,17 +160,20 @@ def main() -> int:
     value = args.batch * steps / dt
     step_bytes = weight_bytes(cfg) + args.batch * mean_ctx * kv_bytes_per_token(cfg)
     achieved = step_bytes / (dt / steps)
+    rs = cfg.rope_scaling
+    rope_text = "none" if rs is None else (f"llama3 factor {rs.factor:g} low {rs.low_freq_factor:g} high "
+                                           f"{rs.high_freq_factor:g} orig {rs.original_max_position_embeddings}")
     out = {
-        "metric": f"decode tokens/s, Llama-3.2-1B shape, batch {args.batch}, context {args.context}, one MI355X",
+        "metric": f"decode tokens/s, {shape_name} shape, batch {args.batch}, context {args.context}, one MI355X",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
-        "config": {"model": "llama-3.2-1b-shape", "global_batch": args.batch, "seq_len": args.context,
-                   "parallelism": "single-gpu", "layers": args.layers, "layers_full": full_layers,
+        "config": {"model": shape_name.lower() + "-shape", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single-gpu", "layers": cfg.num_hidden_layers, "layers_full": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "page_size": page, "tied_embeddings": True, "rope_theta": cfg.rope_theta,
-                   "rope_scaling": "llama3 factor 32 low 1 high 4 orig 8192", "prefill_tokens": 2048},
+                   "page_size": page, "tied_embeddings": cfg.tie_word_embeddings, "rope_theta": cfg.rope_theta,
+                   "rope_scaling": rope_text, "prefill_tokens": 2048},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
     }

@@ -289,3 +289,88 @@ def test_eos_stops_a_request():
     runner = FakeRunner(num_pages=32, page_size=4)
     Scheduler(runner, FakeSampler(), EngineConfig(page_size=4, num_pages=32, max_context=128), eos_token_ids=[eos]).run([r])
     assert r.generated == want[: want.index(eos) + 1]
+
+
+# ---------------------------------------------------------------------------------------------
+# the scheduler one step ahead of the host: a runner whose tokens come back one step late
+# ---------------------------------------------------------------------------------------------
+class FakeHandle:
+    def __init__(self, toks):
+        self._toks, self.read = toks, False
+
+    def tokens(self):
+        self.read = True
+        return list(self._toks)
+
+
+class FakeAheadRunner(FakeRunner):
+    """Launches steps ahead as the real runner does: a request's token may be left out (None) and
+    is then the one the previous launch drew for it, which this runner keeps "on the device"."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.drawn = {}                         # request -> token drawn by the previous launch
+        self.launched_ahead = 0
+        self.handles = []
+
+    def can_decode_async(self, n):
+        return False                            # no graphs here: every step takes the general launch
+
+    def can_launch_ahead(self):
+        return True
+
+    def decode_launch(self, *a, **kw):          # its presence switches the scheduler's pipeline on
+        raise AssertionError("not used without graphs")
+
+    def step_launch(self, req_ids, tokens, samples, temperatures, keys):
+        if self.handles and not self.handles[-1].read:
+            self.launched_ahead += 1            # launched while the step before is still unread
+        segs = []
+        for r, toks, smp in zip(req_ids, tokens, samples):
+            if toks[0] is None:
+                assert len(toks) == 1 and r in self.drawn, "a token left to the device must have been drawn by the launch before"
+                toks = [self.drawn[r]]
+            segs.append(Segment(r, list(toks), [len(toks) - 1] if smp else []))
+        out = self.step(segs)
+        self.drawn = {r: t for r, t in zip([r for r, smp in zip(req_ids, samples) if smp], out)}
+        assert len(temperatures) == len(keys) == len(out)
+        h = FakeHandle(out)
+        self.handles.append(h)
+        return h
+
+
+class FakeSeededSampler(FakeSampler):
+    seed = 7                                    # the pipeline draws on the device and needs the keys' seed
+
+
+@pytest.mark.parametrize("admission", ["reserve", "optimistic"])
+@pytest.mark.parametrize("budget,chunk,pages", [(2048, 2048, 64), (16, 8, 64), (7, 5, 64), (16, 8, 14)])
+def test_steps_launched_ahead_give_every_request_its_own_tokens(admission, budget, chunk, pages):
+    rng = random.Random(5)
+    reqs = make_requests(rng, 14, max_prompt=30, max_new=12)
+    reqs[2].max_new_tokens = 1
+    runner = FakeAheadRunner(num_pages=pages, page_size=4, max_context=56)
+    cfg = EngineConfig(max_tokens_per_step=budget, prefill_chunk=chunk, admission=admission, max_context=56,
+                       page_size=4, num_pages=pages)
+    sched = Scheduler(runner, FakeSeededSampler(), cfg)
+    assert sched.async_decode
+    done = sched.run(reqs)
+    for r in done:
+        assert r.error is None and r.generated == alone(r.prompt, r.max_new_tokens), r.req_id
+    assert runner.launched_ahead > 0 and all(h.read for h in runner.handles)
+    assert all(sum(n for _, n in st) <= budget for st in runner.steps)
+    assert runner.cache.free_pages() == pages and not runner.cache.live_requests()
+    if admission == "optimistic" and pages == 14:
+        assert any(r.preemptions for r in done)             # recomputed from prompt + resolved tokens
+
+
+def test_stop_tokens_keep_the_host_in_step():
+    """Whether a request ends may then depend on a token: the scheduler reads every step's tokens
+    before it plans the next, and never asks the runner to launch ahead."""
+    stop = alone([4, 5], 3)[2]
+    runner = FakeAheadRunner(num_pages=64, page_size=4)
+    sched = Scheduler(runner, FakeSeededSampler(), EngineConfig(page_size=4, num_pages=64, max_context=256),
+                      eos_token_ids=[stop])
+    assert not sched.async_decode
+    out = sched.run([GenerationRequest(1, [4, 5], 6)])
+    assert out[0].generated == alone([4, 5], 3) and runner.handles == []

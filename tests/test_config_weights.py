@@ -180,3 +180,15 @@ def test_engine_refuses_to_run_without_a_gpu():
     from serve_amd.engine.engine import Engine
     with pytest.raises(RuntimeError, match="GPU"):
         Engine.from_config(util.TINY_A, 0)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The engine runs on one GPU: for another count bench.py prints one line that says so and
+    exits with 2 (before it touches torch or the GPU)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                          text=True, timeout=60)
+    assert proc.returncode == 2
+    assert len(proc.stdout.strip().splitlines()) == 1 and "one GPU" in proc.stdout

@@ -563,7 +563,10 @@ static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int 
   // (the choices below are the best of a sweep over RT, KS and KU at the Llama-3.2-1B sizes; the
   // sweep is flat: every shape that fills the chip runs at about 3 us + bytes / 5.3 TB/s)
   if constexpr (EPI == EPI_QKV_ROPE) GO(1, 1, 8, 8);
-  if constexpr (EPI == EPI_SWIGLU) GO(2, 1, 2, 8);
+  if constexpr (EPI == EPI_SWIGLU) {
+    if (K >= 4096) GO(2, 1, 4, 8);   // a long inner dimension: four waves share it
+    GO(2, 1, 2, 8);
+  }
   if constexpr (EPI == EPI_PLAIN) {
     if (N >= 8192) GO(2, 1, 2, 8);
     if (parts > 1) GO(1, 1, 2, 8);   // K is already cut across workgroups: 2 waves each

@@ -273,7 +273,7 @@ def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tor
 def split_k_parts(M: int, N: int, K: int) -> int:
     """Into how many slices the inner dimension of a few-row product is cut across workgroups so
     that a matrix with few rows still fills the chip: 1 means no cut.  Up to 16 rows a workgroup
-    takes 16 weight rows (about 512 workgroups wanted, slices of at least 256); from 17 rows on it
+    takes 16 weight rows (about 1024 workgroups wanted, slices of at least 256); from 17 rows on it
     takes 32 (one workgroup per compute unit wanted, slices of at least 512)."""
     if N >= 8192:
         return 1
@@ -284,7 +284,7 @@ def split_k_parts(M: int, N: int, K: int) -> int:
             parts *= 2
         return parts
     tiles = -(-N // 16)
-    while parts < 4 and tiles * parts < 512 and K // (parts * 2) >= 512:
+    while parts < 4 and tiles * parts < 1024 and K // (parts * 2) >= 512:
         parts *= 2
     return parts
 

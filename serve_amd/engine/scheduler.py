@@ -312,11 +312,11 @@ class Scheduler:
 
     def _launch_step(self, plan: StepPlan) -> None:
         """A step with prompt portions, launched ahead of the host like `_launch_decode`."""
-        from ..sampling.sampler import _signed, row_key
+        from ..sampling.sampler import row_keys
         reqs = plan.requests
         tokens = [r.tokens_between(r.fed, r.fed + n) for r, n in zip(reqs, plan.counts)]
         samplers = [r for r, s in zip(reqs, plan.samples) if s]
-        keys = [_signed(row_key(self.sampler.seed, r.req_id, len(r.generated))) for r in samplers]
+        keys = row_keys(self.sampler.seed, [r.req_id for r in samplers], [len(r.generated) for r in samplers])
         handle = self.runner.step_launch([r.req_id for r in reqs], tokens, plan.samples,
                                          [r.temperature for r in samplers], keys)
         previous, self._inflight = self._inflight, (handle, samplers, [len(r.generated) for r in samplers])
@@ -333,10 +333,10 @@ class Scheduler:
             self._read_back(previous)
 
     def _launch_decode(self, plan: StepPlan) -> None:
-        from ..sampling.sampler import _signed, row_key
+        from ..sampling.sampler import row_keys
         reqs = plan.requests
         tokens = [(r.generated[-1] if r.generated else r.prompt[-1]) for r in reqs]
-        keys = [_signed(row_key(self.sampler.seed, r.req_id, len(r.generated))) for r in reqs]
+        keys = row_keys(self.sampler.seed, [r.req_id for r in reqs], [len(r.generated) for r in reqs])
         handle = self.runner.decode_launch([r.req_id for r in reqs], tokens, [r.temperature for r in reqs], keys)
         previous, self._inflight = self._inflight, (handle, list(reqs), [len(r.generated) for r in reqs])
         self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in reqs], counts=[1] * len(reqs),

@@ -11,6 +11,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -35,6 +36,22 @@ def _signed(u: int) -> int:
     return u - (1 << 64) if u >= (1 << 63) else u
 
 
+def _mix64_np(z: np.ndarray) -> np.ndarray:
+    z = z + np.uint64(0x9E3779B97F4A7C15)
+    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+def row_keys(seed: int, request_ids: Sequence[int], token_indices: Sequence[int]) -> np.ndarray:
+    """`row_key` of many rows at once, as the int64 bit patterns the kernel takes."""
+    with np.errstate(over="ignore"):
+        rid = np.asarray([int(r) & _MASK for r in request_ids], dtype=np.uint64)
+        idx = np.asarray([int(i) & _MASK for i in token_indices], dtype=np.uint64)
+        key = _mix64_np(np.uint64(mix64(seed & _MASK)) ^ rid)
+        return _mix64_np(key ^ idx).view(np.int64)
+
+
 class Sampler:
     def __init__(self, seed: int, device):
         self.seed = int(seed)
@@ -54,8 +71,8 @@ class Sampler:
         else:
             if request_ids is None or token_indices is None or len(request_ids) != R or len(token_indices) != R:
                 raise ValueError("a draw needs the request id and the token index of every row")
-            keys = [_signed(row_key(self.seed, int(r), int(i))) for r, i in zip(request_ids, token_indices)]
+            keys = row_keys(self.seed, request_ids, token_indices)
             t_dev = torch.tensor([float(t) for t in temperatures], dtype=torch.float32, device=logits.device)
-            k_dev = torch.tensor(keys, dtype=torch.int64, device=logits.device)
+            k_dev = torch.from_numpy(keys).to(logits.device)
             ops.sample(logits, t_dev, k_dev, out)
         return out.tolist()

@@ -20,8 +20,6 @@ import os
 import sys
 from typing import Iterable, Optional, TextIO
 
-import numpy as np
-
 from ..config.engine import EngineConfig
 from .batch import Segment
 from .engine import Engine

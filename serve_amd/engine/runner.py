@@ -19,7 +19,7 @@ from ..cache.storage import CacheStorage, bytes_per_page, group_windows
 from ..config.engine import EngineConfig
 from ..models.model import Model
 from ..parts.base import Runtime
-from .batch import Segment, StepContext, StepLayout, build_step, context_from, plan_step
+from .batch import Segment, StepLayout, build_step, context_from, plan_step
 
 # padded batch sizes for which decode-only steps are captured into graphs
 GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64, 128, 256)

@@ -10,7 +10,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..config.spec import ModelSpec, PartSpec
-from ..parts.base import KVCacheRequest, LayerCache, ParamRequest, Part, Runtime, StateRequest
+from ..parts.base import KVCacheRequest, LayerCache, Part, Runtime, StateRequest
 from ..registry import get_part
 
 

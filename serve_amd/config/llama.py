@@ -48,6 +48,11 @@ class Llama3RopeScaling:
         return d
 
 
+def _no_scaling(scaling: Optional[Dict[str, Any]]) -> bool:
+    """config.json says "no scaling" as null or as {"rope_type": "default"}."""
+    return scaling is None or scaling.get("rope_type", scaling.get("type")) == "default"
+
+
 @dataclass(frozen=True)
 class LlamaConfig:
     """config.json of `LlamaForCausalLM`.  Field names are the file's keys."""
@@ -105,7 +110,7 @@ class LlamaConfig:
             head_dim=int(head_dim),
             rms_norm_eps=float(d.get("rms_norm_eps", 1e-5)),
             rope_theta=float(d.get("rope_theta", 10000.0)),
-            rope_scaling=None if scaling is None else Llama3RopeScaling.from_hf_dict(scaling),
+            rope_scaling=None if _no_scaling(scaling) else Llama3RopeScaling.from_hf_dict(scaling),
             max_position_embeddings=int(d.get("max_position_embeddings", 131072)),
             tie_word_embeddings=bool(d.get("tie_word_embeddings", False)),
             bos_token_id=d.get("bos_token_id"),

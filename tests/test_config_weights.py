@@ -192,3 +192,19 @@ def test_bench_refuses_more_than_one_gpu():
                           text=True, timeout=60)
     assert proc.returncode == 2
     assert len(proc.stdout.strip().splitlines()) == 1 and "one GPU" in proc.stdout
+
+
+def test_config_json_of_a_checkpoint_with_all_its_keys():
+    """config.json as checkpoints ship it: keys the engine has no use for are ignored, absent
+    head_dim and num_key_value_heads take their defaults, "default" rope scaling means none."""
+    hf = {"architectures": ["LlamaForCausalLM"], "attention_bias": False, "attention_dropout": 0.0,
+          "bos_token_id": 128000, "eos_token_id": [128001, 128008], "hidden_act": "silu", "hidden_size": 96,
+          "initializer_range": 0.02, "intermediate_size": 200, "max_position_embeddings": 4096, "mlp_bias": False,
+          "model_type": "llama", "num_attention_heads": 6, "num_hidden_layers": 2, "pretraining_tp": 1,
+          "rms_norm_eps": 1e-05, "rope_scaling": {"rope_type": "default"}, "rope_theta": 500000.0,
+          "torch_dtype": "bfloat16", "transformers_version": "4.45.0", "use_cache": True, "vocab_size": 300}
+    cfg = LlamaConfig.from_hf_dict(hf)
+    assert (cfg.head_dim, cfg.num_key_value_heads, cfg.rope_scaling, cfg.tie_word_embeddings) == (16, 6, None, False)
+    hf["rope_scaling"] = {"type": "linear", "factor": 2.0}
+    with pytest.raises(Exception, match="linear"):
+        LlamaConfig.from_hf_dict(hf)

@@ -10,9 +10,10 @@
 // partial (m, l, O) are merged with the running maximum (the reference's merge,
 // attn_decode.py:341-348, has none and is switched off).
 //
-// Work item of one wave: (segment, KV head, tile of 16*NT "rows", split of the key range).  The
-// rows of a segment are its (token, query head of the group) pairs, row = token * G + head_in_group,
-// so the G heads that share a KV head share every K and V load.
+// The rows of a segment are its (token, query head of the group) pairs, row = token * G +
+// head_in_group, so the G heads that share a KV head share every K and V load.  Two kernels: one
+// wave per (segment, KV head, split of the key range) for single decoded tokens, workgroups that
+// share K and V through LDS for prompt portions.
 //
 // MFMA use (v_mfma_f32_16x16x32_bf16: D[i][j] += sum_k A[i][k] B[k][j]; lane l holds A row l%16,
 // B column l%16, k-slots 8*(l/16)..+7, and D[4*(l/16)+r][l%16]):
@@ -67,14 +68,14 @@ __device__ __forceinline__ float max_across_groups(float x) {
 struct Masked { static constexpr bool value = true; };
 struct Unmasked { static constexpr bool value = false; };
 
-// NT: column tiles (16 query rows each) per wave.  PM: how keys map to pages:
+// Single decoded tokens (at most 16 rows per KV head and segment): one wave per (segment, KV head,
+// split of the key range), K and V straight from the cache into registers.  PM: how keys map to pages:
 //   0  any page size that is a multiple of 4: division per key, 8-byte value runs;
 //   1  a power of two of at least 8: shift, 16-byte value runs; a block of 32 keys spans up to four
 //      pages and each lane picks its own;
 //   2  a power of two of at least 32: a block lies in one page, and every address is a scalar base
 //      plus a constant of the lane.
-// One tile of one (segment, KV head, split): everything a wave does.
-template <int NT, int PM>
+template <int PM>
 __device__ __forceinline__ void attention_tile(
     const int tile, const int seg, const int hk, const int sp, const int q_begin, const int q_len,
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -82,6 +83,7 @@ __device__ __forceinline__ void attention_tile(
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ ctx_len, int Hq, int Hk,
     int page_size, int page_shift, float scale_log2e, int window, int num_splits,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int NT = 1;                                     // column tiles of 16 rows per wave
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
   const int c = lane & 15;
@@ -333,32 +335,11 @@ __device__ __forceinline__ void attention_tile(
         acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pf[n].v, acc[dt][n], 0, 0, 0);
   };
 
-  // Three buffers in turn: the loads of the next two blocks are in flight while one is computed
-  // (two buffers, one block in flight, for prompt tiles of head sizes above 64, whose blocks are
-  // twice as large and would push the registers over the edge).
+  // Three buffers in turn: the loads of the next two blocks are in flight while one is computed.
   // The loads carry no conditions: a block beyond the last is read from clamped keys and pages and
   // never used.  With a branch around them the compiler no longer knows how many loads are in
   // flight where a block's data is awaited, and waits for all of them, the newest included.
-  if (b0 < b1 && HD > 64 && NT > 1) {
-    Block buf_a, buf_b;
-    prefetch_pages(b0);
-    load_block(b0, buf_a);
-    int kb = b0;
-    for (; kb + 2 <= b1; kb += 2) {
-      if (kb >= full_lo && kb + 1 <= full_hi) {
-        load_block(kb + 1, buf_b);
-        compute(kb, buf_a, Unmasked{});
-        load_block(kb + 2, buf_a);
-        compute(kb + 1, buf_b, Unmasked{});
-      } else {
-        load_block(kb + 1, buf_b);
-        compute(kb, buf_a, Masked{});
-        load_block(kb + 2, buf_a);
-        compute(kb + 1, buf_b, Masked{});
-      }
-    }
-    if (kb < b1) compute(kb, buf_a, Masked{});
-  } else if (b0 < b1) {
+  if (b0 < b1) {
     Block buf_a, buf_b, buf_c;
     prefetch_pages(b0);
     load_block(b0, buf_a);
@@ -419,10 +400,7 @@ __device__ __forceinline__ void attention_tile(
   }
 }
 
-// A wave takes tile w of its (segment, KV head).  With PAIR it takes tile ntiles-1-w as well: under
-// the causal mask tile t reads keys up to about t's end, so the two together are always one full
-// context long and all waves of a prompt finish at about the same time.
-template <int NT, int PM, bool PAIR>
+template <int PM>
 __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
@@ -435,22 +413,513 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int sp = blockIdx.z - seg * num_splits;
   const int q_begin = cu_q[seg];
   const int q_len = cu_q[seg + 1] - q_begin;
-  if (!PAIR) {
-    attention_tile<NT, PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
-                             max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
-                             part_o, part_ml);
-    return;
+  attention_tile<PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table, max_pages,
+                     ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits, part_o, part_ml);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prompt portions (more than 16 rows in a segment).  A workgroup of eight waves takes TW tiles of
+// 32 rows, next to one another in the segment, and walks over the keys in stages of KW * KB blocks
+// of 32 keys (TW * KW = 8).  All eight waves fetch a stage together, 16 bytes a thread at a time,
+// into registers (up to two stages ahead) and from there into LDS one stage ahead; then wave
+// (tw, kw) multiplies tile tw with the kw-th run of KB blocks of the stage, reading K and V^T from
+// LDS in the lane order of the matrix instruction, with one softmax update (maximum, rescaling of
+// O) for the 32 * KB keys.  The KW waves of a tile hold partial (m, l, O), merged through LDS at
+// the end.  K and V cross the chip's caches once per 32 * TW rows instead of once per wave.
+//
+// What the time goes to is the number of instructions a SIMD has to issue: measured on this chip,
+// a SIMD whose two waves keep the vector unit busy gains little from matrix instructions of the
+// other wave running beside them (288 vector + 32 matrix instructions: 429 ns + 229 ns apart,
+// 589 ns together), and an exponential costs about three and a half ordinary vector instructions.
+// Hence one softmax update per 64 keys, three-way maxima, row sums taken by the matrix cores, O
+// rescaled only when a maximum has moved, and page addresses that are a constant plus a product.
+//
+// The work per stage is the same straight line of code for every wave and stage: a block that is
+// partly or wholly invisible to the tile (the causal edge, the window's edge, beyond the tile's
+// last key) has its scores masked under a branch that touches nothing else, and contributes
+// p = 0.  A branch around the matrix products themselves would make the compiler copy O at every
+// stage.
+//
+// LDS of a stage: K as [key][16-byte slot] with rows of 128 bytes (256 above head size 64), slot
+// s of key row r stored at s ^ ((r & 3) | ((r >> 1) & 4)): the eight lanes that read together
+// (c = 0..7 -> rows 0..3, 8..11 of a block, one slot) then fall into eight different 16-byte bank
+// groups, and so do the eight threads that write one key's row.  V^T as [block][dim][4 runs of
+// 8 keys], run g of dim d at g ^ ((d >> 1) & 3).
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int log2_of(int x) { return x <= 1 ? 0 : 1 + log2_of(x / 2); }
+
+template <int KW>
+struct PromptShape {
+  static constexpr int TW = 8 / KW;                        // tiles of 32 rows per workgroup
+  static constexpr int KB = HD <= 64 ? 2 : 1;              // blocks of 32 keys per wave and stage
+  static constexpr int BLOCKS = KW * KB;
+  static constexpr int KEYS = 32 * BLOCKS;                 // keys per stage
+  static constexpr int K_ROW = HD <= 64 ? 128 : 256;       // bytes of a key's row in LDS
+  static constexpr int K_BYTES = KEYS * K_ROW;
+  static constexpr int V_BYTES = BLOCKS * HD * 64;
+  static constexpr int STAGE = K_BYTES + V_BYTES;
+  static constexpr int STAGES = 3 * STAGE <= 144 * 1024 ? 3 : 2;
+  static constexpr int LDS_BYTES = STAGES * STAGE;
+  static constexpr int CHUNKS = 4 * BLOCKS * HD;           // 16-byte pieces of K, and of V, per stage
+  static constexpr int PER_THREAD = (CHUNKS + 511) / 512;
+  static constexpr int RING = PER_THREAD <= 2 ? 2 : 1;     // stages held in registers on their way to LDS
+  static constexpr int MERGE_FLOATS = DT * 8 + 4;          // per lane: O, m and l of two column tiles
+  static_assert((KW - 1) * TW * MERGE_FLOATS * 64 * 4 <= LDS_BYTES, "the merge reuses the stages' memory");
+  static_assert(TW * KW == 8, "eight waves");
+};
+
+template <int KW, int PM>
+__global__ __launch_bounds__(512) void prompt_attention_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
+    int window, int num_splits, int pair, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  using S = PromptShape<KW>;
+  constexpr int TW = S::TW, KB = S::KB, NT = 2, PT = S::PER_THREAD;
+  constexpr int VL = PM == 0 ? 2 : 1;                      // loads per 16 bytes of V^T
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tw = wave % TW;
+  const int kw = wave / TW;
+  // neighbours in the grid take different KV heads: with eight of them each of the chip's eight
+  // dies (workgroups are dealt to them in turn) reads one head's keys and values only
+  const int hk = blockIdx.x % Hk;
+  const int item = blockIdx.x / Hk;
+  const int seg = blockIdx.y / num_splits;
+  const int sp = blockIdx.y - seg * num_splits;
+  const int q_begin = cu_q[seg];
+  const int q_len = cu_q[seg + 1] - q_begin;
+  const int G = Hq / Hk;
+  const int rows_total = q_len * G;
+  const int ngroups = (rows_total + 32 * TW - 1) / (32 * TW);
+  if (item >= (pair ? (ngroups + 1) / 2 : ngroups)) return;
+  const int ctx = ctx_len[seg];
+  const int ctx_before = ctx - q_len;
+  const int* bt = block_table + (size_t)seg * max_pages;
+  const uint32_t page_bytes = (uint32_t)Hk * page_size * HD * 2;   // of a page of K, and of V (checked by the host)
+  const int last_page = PM == 1 ? (ctx - 1) >> page_shift : (ctx - 1) / page_size;
+  const char* k_base = reinterpret_cast<const char*>(k_pages);
+  const char* v_base = reinterpret_cast<const char*>(v_pages);
+
+  // ---- what this thread fetches of every stage ---------------------------------------------
+  // With a power-of-two page size a stage begins at a multiple of its own length or of the page
+  // size, so a key's place in its page is a constant of the thread plus (stage begin mod page):
+  // k_off / v_off hold the constant, in bytes from the page's begin.  Keys beyond the context are
+  // read from the last page, at their own place in it, and are never visible.
+  int k_key[PT], k_seg[PT], k_off[PT], k_lds[PT], v_run[PT], v_dim[PT], v_off[PT], v_lds[PT];
+  bool fetches[PT];
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int raw = tid + i * 512;
+    fetches[i] = raw < S::CHUNKS;
+    const int ch = min(raw, S::CHUNKS - 1);
+    k_key[i] = ch / (HD / 8);
+    k_seg[i] = ch - k_key[i] * (HD / 8);
+    k_lds[i] = k_key[i] * S::K_ROW + ((k_seg[i] ^ ((k_key[i] & 3) | ((k_key[i] >> 1) & 4))) << 4);
+    if (PM == 1) {
+      // consecutive threads take consecutive 16 bytes of a page's [D, page_size] values: runs
+      // of 8 keys along a dim, then the next dim
+      const int rs = min(page_shift - 3, log2_of(4 * S::BLOCKS));   // a page's piece in the stage: 2^rs runs
+      const int piece = (ch >> rs) / HD;
+      const int within = ch - ((piece * HD) << rs);
+      v_dim[i] = within >> rs;
+      v_run[i] = (piece << rs) + (within & ((1 << rs) - 1));
+      k_off[i] = (((hk * page_size + (k_key[i] & (page_size - 1))) * HD) + k_seg[i] * 8) * 2;
+      v_off[i] = ((hk * HD + v_dim[i]) * page_size + ((v_run[i] * 8) & (page_size - 1))) * 2;
+    } else {
+      v_run[i] = ch / HD;
+      v_dim[i] = ch - v_run[i] * HD;
+      k_off[i] = v_off[i] = 0;
+    }
+    v_lds[i] = S::K_BYTES + ((((v_run[i] >> 2) * HD + v_dim[i]) * 4 + ((v_run[i] & 3) ^ ((v_dim[i] >> 1) & 3))) << 4);
   }
-  const int ntiles = (q_len * (Hq / Hk) + 16 * NT - 1) / (16 * NT);
-  if (w >= (ntiles + 1) / 2) return;                                  // the second half is done by pairing
-  attention_tile<NT, PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
-                           max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
-                           part_o, part_ml);
-  const int other = ntiles - 1 - w;
-  if (other > w)
-    attention_tile<NT, PM>(other, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
-                             max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits,
-                             part_o, part_ml);
+  struct Ring {
+    u32x4_t k[PT], v[PT];
+  };
+  // page ids of a stage, fetched one step before the stage's keys and values are
+  auto lookup = [&](int sb, int (&pk)[PT], int (&pv)[PT * VL]) __attribute__((always_inline)) {
+    const int key0 = sb * S::KEYS;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      if (PM == 1) {
+        pk[i] = bt[min((key0 + k_key[i]) >> page_shift, last_page)];
+        pv[i] = bt[min((key0 + v_run[i] * 8) >> page_shift, last_page)];
+      } else {
+        pk[i] = bt[min((key0 + k_key[i]) / page_size, last_page)];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) pv[i * VL + h] = bt[min((key0 + v_run[i] * 8 + 4 * h) / page_size, last_page)];
+      }
+    }
+  };
+  // The loads carry no conditions: a stage beyond the last is read from the last page and never used.
+  auto issue = [&](int sb, const int (&pk)[PT], const int (&pv)[PT * VL], Ring& r) __attribute__((always_inline)) {
+    const int key0 = sb * S::KEYS;
+    if (PM == 1) {
+      const int in_page = key0 & (page_size - 1);           // 0 unless a page holds several stages
+      const char* kb = k_base + (size_t)in_page * (HD * 2);
+      const char* vb = v_base + (size_t)in_page * 2;
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        r.k[i] = *reinterpret_cast<const u32x4_t*>(kb + ((uint64_t)(uint32_t)max(pk[i], 0) * page_bytes + (uint32_t)k_off[i]));
+        r.v[i] = *reinterpret_cast<const u32x4_t*>(vb + ((uint64_t)(uint32_t)max(pv[i], 0) * page_bytes + (uint32_t)v_off[i]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        const int key = key0 + k_key[i];
+        const int off = key % page_size;
+        r.k[i] = *reinterpret_cast<const u32x4_t*>(k_base + (uint64_t)(uint32_t)max(pk[i], 0) * page_bytes +
+                                                   ((size_t)(hk * page_size + off) * HD + k_seg[i] * 8) * 2);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int run = key0 + v_run[i] * 8 + 4 * h;
+          const u32x2_t half = *reinterpret_cast<const u32x2_t*>(
+              v_base + (uint64_t)(uint32_t)max(pv[i * VL + h], 0) * page_bytes +
+              ((size_t)(hk * HD + v_dim[i]) * page_size + run % page_size) * 2);
+          r.v[i][2 * h] = half[0];
+          r.v[i][2 * h + 1] = half[1];
+        }
+      }
+    }
+  };
+  // registers -> LDS.  Values of keys at or beyond the end of the context hold whatever the page
+  // held before: their probability is 0, and 0 times such a value must stay 0, so they are zeroed.
+  auto stash = [&](int sb, int stage, const Ring& r) __attribute__((always_inline)) {
+    unsigned char* st = smem + stage * S::STAGE;
+    const int key0 = sb * S::KEYS;
+    const bool at_end = key0 + S::KEYS > ctx;               // the same for every thread
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      u32x4_t v = r.v[i];
+      if (at_end) {
+        const int first = key0 + v_run[i] * 8;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          v[e] &= (first + 2 * e < ctx ? 0x0000ffffu : 0u) | (first + 2 * e + 1 < ctx ? 0xffff0000u : 0u);
+      }
+      if (S::CHUNKS % 512 == 0 || fetches[i]) {
+        *reinterpret_cast<u32x4_t*>(st + k_lds[i]) = r.k[i];
+        *reinterpret_cast<u32x4_t*>(st + v_lds[i]) = v;
+      }
+    }
+  };
+
+  // ---- where this lane reads its operands in a stage ----------------------------------------
+  const int krow = kw * KB * 32 + 8 * (c >> 2) + (c & 3);   // key row of tile 0 of the wave's first block
+  const int kswz = c & 7;                                    // the row's slot mask: (r & 3) | ((r >> 1) & 4), all tiles
+  const int ka0 = krow * S::K_ROW + ((g ^ kswz) << 4);       // dims 0..31 (and 64..95, 128 bytes on)
+  const int ka1 = krow * S::K_ROW + (((4 + g) ^ kswz) << 4); // dims 32..63 (and 96..127)
+  const int va = S::K_BYTES + (((kw * KB * HD + c) * 4 + (g ^ ((c >> 1) & 3))) << 4);
+  Frag ones;
+  ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);   // bf16 1.0 throughout
+
+  for (int pass = 0; pass < 2; ++pass) {
+    const int group = pass == 0 ? item : ngroups - 1 - item;
+    if (pass == 1) {
+      if (!pair || group <= item) break;
+      __syncthreads();                                      // the first group's merge has been read
+    }
+    // the workgroup's range of stages, and this split's part of it
+    const int r0g = group * (32 * TW);
+    const int hi_key_g = ctx_before + min(rows_total - 1, r0g + 32 * TW - 1) / G;
+    const int lo_key_g = window > 0 ? max(0, ctx_before + r0g / G - window + 1) : 0;
+    const int sb_lo = lo_key_g / S::KEYS;
+    const int sb_hi = hi_key_g / S::KEYS;
+    const int per = (sb_hi - sb_lo + num_splits) / num_splits;
+    const int s0 = __builtin_amdgcn_readfirstlane(sb_lo + sp * per);
+    const int nsb = __builtin_amdgcn_readfirstlane(max(0, min(sb_hi + 1, s0 + per) - s0));
+    // this wave's tile (a tile beyond the segment's rows computes the last row over again and
+    // writes nothing)
+    const int r0 = r0g + tw * 32;
+    const bool active = r0 < rows_total;
+    const int j_lo = min(r0, rows_total - 1) / G;
+    const int j_hi = min(rows_total - 1, r0 + 31) / G;
+    // blocks full_lo .. full_hi are visible as a whole to every row of the tile
+    const int full_hi = __builtin_amdgcn_readfirstlane((ctx_before + j_lo - 31) >> 5);
+    const int full_lo = window > 0 ? __builtin_amdgcn_readfirstlane(((ctx_before + j_hi - window) >> 5) + 1) : 0;
+
+    int qpos[NT], tok[NT], head[NT];
+    bool rvalid[NT];
+    Frag qf[NT][DC];
+    float m[NT], m_raw[NT];
+    floatx4_t lsum[NT];                                     // every element: the sum of p over all keys so far
+    floatx4_t acc[DT][NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      const int row = r0 + n * 16 + c;
+      rvalid[n] = row < rows_total;
+      const int rowc = min(row, rows_total - 1);
+      const int j = rowc / G;
+      tok[n] = q_begin + j;
+      head[n] = hk * G + (rowc - j * G);
+      qpos[n] = ctx_before + j;
+      const bf16_t* qp = q + (size_t)tok[n] * q_stride + (size_t)head[n] * HD;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        qf[n][dc].u = make_uint4(0, 0, 0, 0);
+        if (dc * 32 + g * 8 < HD) qf[n][dc].u = *reinterpret_cast<const uint4*>(qp + dc * 32 + g * 8);
+      }
+      m[n] = m_raw[n] = -INFINITY;
+      lsum[n] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[dt][n] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+    }
+
+    struct Scores {
+      floatx4_t v[KB][2][NT];
+    };
+    // S^T = K Q^T for this wave's KB blocks of LDS stage `stage`
+    auto qk = [&](int stage, Scores& sc) __attribute__((always_inline)) {
+      const unsigned char* st = smem + stage * S::STAGE;
+      auto& s = sc.v;
+#pragma unroll
+      for (int h = 0; h < KB; ++h) {
+        Frag kf[2][DC];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int dc = 0; dc < DC; ++dc) {
+            kf[t][dc].u = *reinterpret_cast<const uint4*>(st + ((dc & 1) ? ka1 : ka0) + (h * 32 + t * 4) * S::K_ROW +
+                                                          (dc >> 1) * 128);
+            // dims beyond the head size were never written: they must read as 0, not as what LDS held
+            if (HD % 32 != 0 && dc == DC - 1 && dc * 32 + g * 8 >= HD) kf[t][dc].u = make_uint4(0, 0, 0, 0);
+          }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int n = 0; n < NT; ++n) {
+            s[h][t][n] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc)
+              s[h][t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][dc].v, qf[n][dc].v, s[h][t][n], 0, 0, 0);
+          }
+      }
+    };
+    // blocks kb .. kb + KB - 1 of the keys: softmax update with their scores, O^T += V^T P^T with
+    // the values of LDS stage `stage`
+    auto softmax_pv = [&](int kb, int stage, Scores& sc) __attribute__((always_inline)) {
+      const unsigned char* st = smem + stage * S::STAGE;
+      auto& s = sc.v;
+      // some key of these blocks is invisible to some row: the causal edge, the window's edge, a
+      // block beyond the tile's last key
+      if (kb < full_lo || kb + KB - 1 > full_hi) {
+#pragma unroll
+        for (int h = 0; h < KB; ++h)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int key = ((kb + h) << 5) + 8 * g + 4 * t + r;
+                const bool vis = key <= qpos[n] && (window <= 0 || key > qpos[n] - window);
+                s[h][t][n][r] = vis ? s[h][t][n][r] : -INFINITY;
+              }
+      }
+      // online softmax over this lane's 8 * KB keys per column, shared across the 4 lane groups.
+      // The scale is positive, so the maximum is taken on the raw scores and the scale is applied
+      // inside the exponent: p = 2^(s * scale - m).  Chains of dependent operations are kept short
+      // (four running maxima; the row sums l come from the matrix cores, see below): a wave waits
+      // several cycles for a result it has just asked for.
+      Frag pf[KB][NT];
+      float alpha[NT];
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        // two chains of three-way maxima over the lane's scores and the maximum so far (kept unscaled
+        // in m_raw for this), then across the four lane groups
+        float ma = fmaxf(fmaxf(m_raw[n], s[0][0][n][0]), s[0][0][n][1]);
+        ma = fmaxf(fmaxf(ma, s[0][0][n][2]), s[0][0][n][3]);
+        float mb = fmaxf(fmaxf(s[0][1][n][0], s[0][1][n][1]), s[0][1][n][2]);
+#pragma unroll
+        for (int h = 1; h < KB; ++h) {
+          ma = fmaxf(fmaxf(ma, s[h][0][n][0]), s[h][0][n][1]);
+          ma = fmaxf(fmaxf(ma, s[h][0][n][2]), s[h][0][n][3]);
+          mb = fmaxf(fmaxf(mb, s[h][1][n][0]), s[h][1][n][1]);
+          mb = fmaxf(fmaxf(mb, s[h][1][n][2]), s[h][1][n][3]);
+        }
+        m_raw[n] = max_across_groups(fmaxf(fmaxf(ma, mb), s[0][1][n][3]));
+        const float m_new = m_raw[n] * scale_log2e;
+        // a row that has seen no visible key yet keeps m = -inf
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        alpha[n] = __builtin_amdgcn_exp2f(m[n] - m_safe);
+        m[n] = m_new;
+#pragma unroll
+        for (int h = 0; h < KB; ++h)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[h][t][n][r] = fmaf(s[h][t][n][r], scale_log2e, -m_safe);
+#pragma unroll
+        for (int h = 0; h < KB; ++h)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[h][t][n][r] = __builtin_amdgcn_exp2f(s[h][t][n][r]);
+#pragma unroll
+        for (int h = 0; h < KB; ++h)
+          pf[h][n].u = make_uint4(pack2bf(s[h][0][n][0], s[h][0][n][1]), pack2bf(s[h][0][n][2], s[h][0][n][3]),
+                                  pack2bf(s[h][1][n][0], s[h][1][n][1]), pack2bf(s[h][1][n][2], s[h][1][n][3]));
+      }
+      // the running maximum rarely moves after the first stages: O and l are rescaled only when it
+      // has, for some row of the wave
+      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.f || alpha[1] != 1.f) != 0) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          lsum[n] *= alpha[n];
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) acc[dt][n] *= alpha[n];
+        }
+      }
+      // O^T += V^T P^T, and l += 1^T P^T: a product with a tile of ones sums p over the keys of the
+      // block (as it was rounded to bf16, which is what multiplies V), in every row of the result
+#pragma unroll
+      for (int h = 0; h < KB; ++h) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+          lsum[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[h][n].v, lsum[n], 0, 0, 0);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          Frag vf;
+          vf.u = *reinterpret_cast<const uint4*>(st + va + (h * HD + dt * 16) * 64);
+#pragma unroll
+          for (int n = 0; n < NT; ++n)
+            acc[dt][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[h][n].v, acc[dt][n], 0, 0, 0);
+        }
+      }
+    };
+
+    if (nsb > 0) {
+      int pk[PT], pv[PT * VL];
+      Ring ra, rb;
+      lookup(s0, pk, pv);
+      issue(s0, pk, pv, ra);
+      lookup(s0 + 1, pk, pv);
+      stash(s0, 0, ra);
+      // one step: stage i + 1 goes from its registers to LDS, the registers are filled again with
+      // the stage RING steps later, then stage i is multiplied
+      int stage = 0;
+      auto step = [&](int i, Ring& r) __attribute__((always_inline)) {
+        const int next = stage + 1 == S::STAGES ? 0 : stage + 1;
+        stash(s0 + i + 1, next, r);
+        issue(s0 + i + 1 + S::RING, pk, pv, r);
+        lookup(s0 + i + 2 + S::RING, pk, pv);
+        __syncthreads();
+        Scores sc;
+        qk(stage, sc);
+        softmax_pv(((s0 + i) * KW + kw) * KB, stage, sc);
+        if (S::STAGES == 2) __syncthreads();
+        stage = next;
+      };
+      if (S::RING == 2) {
+        issue(s0 + 1, pk, pv, rb);
+        lookup(s0 + 2, pk, pv);
+        issue(s0 + 2, pk, pv, ra);
+        lookup(s0 + 3, pk, pv);
+        int i = 0;
+        for (; i + 2 <= nsb; i += 2) {
+          step(i, rb);
+          step(i + 1, ra);
+        }
+        if (i < nsb) step(i, rb);
+      } else {
+        issue(s0 + 1, pk, pv, ra);
+        lookup(s0 + 2, pk, pv);
+        for (int i = 0; i < nsb; ++i) step(i, ra);
+      }
+    }
+
+    // ---- the KW waves of a tile merge through LDS, wave kw = 0 writes ---------------------------
+    float lt[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) lt[n] = lsum[n][0];
+    __syncthreads();                                        // every wave is done with the stages
+    float* mg = reinterpret_cast<float*>(smem);
+    if (kw > 0 && active) {
+      float* mine = mg + (size_t)((kw - 1) * TW + tw) * S::MERGE_FLOATS * 64 + lane;
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        mine[(n * 2) * 64] = m[n];
+        mine[(n * 2 + 1) * 64] = lt[n];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) mine[(4 + (dt * NT + n) * 4 + r) * 64] = acc[dt][n][r];
+      }
+    }
+    __syncthreads();
+    if (kw > 0 || !active) continue;
+#pragma unroll
+    for (int o = 1; o < KW; ++o) {
+      const float* other = mg + (size_t)((o - 1) * TW + tw) * S::MERGE_FLOATS * 64 + lane;
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const float mo = other[(n * 2) * 64];
+        const float lo = other[(n * 2 + 1) * 64];
+        const float mm = fmaxf(m[n], mo);
+        const float wa = m[n] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[n] - mm);   // an empty part weighs 0
+        const float wb = mo == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mo - mm);
+        m[n] = mm;
+        lt[n] = lt[n] * wa + lo * wb;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            acc[dt][n][r] = acc[dt][n][r] * wa + other[(4 + (dt * NT + n) * 4 + r) * 64] * wb;
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      if (!rvalid[n]) continue;
+      if (num_splits == 1) {
+        const float inv = 1.f / lt[n];
+        bf16_t* op = out + ((size_t)tok[n] * Hq + head[n]) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          uint2 w;
+          w.x = pack2bf(acc[dt][n][0] * inv, acc[dt][n][1] * inv);
+          w.y = pack2bf(acc[dt][n][2] * inv, acc[dt][n][3] * inv);
+          *reinterpret_cast<uint2*>(op + dt * 16 + 4 * g) = w;
+        }
+      } else {
+        const size_t slot = ((size_t)tok[n] * Hq + head[n]) * num_splits + sp;
+        float* po = part_o + slot * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          *reinterpret_cast<float4*>(po + dt * 16 + 4 * g) =
+              make_float4(acc[dt][n][0], acc[dt][n][1], acc[dt][n][2], acc[dt][n][3]);
+        if (g == 0) {
+          part_ml[slot * 2] = m[n];
+          part_ml[slot * 2 + 1] = lt[n];
+        }
+      }
+    }
+  }
+}
+
+template <int KW, int PM>
+static int launch_prompt(dim3 grid, hipStream_t stream, const bf16_t* q, int q_stride, bf16_t* out,
+                         const bf16_t* k_pages, const bf16_t* v_pages, const int* block_table, int max_pages,
+                         const int* cu_q, const int* ctx_len, int Hq, int Hk, int page_size, int page_shift,
+                         float scale_log2e, int window, int num_splits, int pair, float* part_o, float* part_ml) {
+  constexpr int lds = PromptShape<KW>::LDS_BYTES;
+  static bool sized = false;          // more than 64 KB of LDS has to be asked for, once per kernel
+  if (!sized) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prompt_attention_kernel<KW, PM>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    sized = true;
+  }
+  hipLaunchKernelGGL((prompt_attention_kernel<KW, PM>), grid, dim3(512), lds, stream, q, q_stride, out, k_pages,
+                     v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e,
+                     window, num_splits, pair, part_o, part_ml);
+  return 0;
 }
 
 // out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s; at most 64 splits.
@@ -497,16 +966,8 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
 
 extern "C" int sa_attention_mfma_head_dim() { return HD; }
 
-// Tiles of 16*nt rows per wave: nt = 1 when a segment has at most 16 rows (decode steps).  Prompt
-// portions take the largest tile the registers hold (fewest reads of K and V) when that still gives
-// every SIMD of the chip a wave, and 32 rows otherwise.
-#if HEAD_DIM <= 64
-#define NT_PREFILL 4
-#else
-#define NT_PREFILL 2
-#endif
-constexpr int WAVES_TO_FILL = 1024;     // 256 compute units x 4 SIMDs
-
+// A step whose segments have at most 16 rows each (single decoded tokens) takes the one-wave kernel,
+// any other the prompt kernel.
 extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, const void* k_pages,
                                        const void* v_pages, const int* block_table, int max_pages,
                                        const int* cu_q, const int* ctx_len, int B, int T, int max_q_len,
@@ -520,43 +981,49 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   if ((long long)B * num_splits > 65535 || Hk > 65535) return SA_ERR_ARG;
   const int G = Hq / Hk;
   const bool small = (long long)max_q_len * G <= 16;
-  // prompt portions: a wave takes tiles w and tiles-1-w, so half as many waves are launched
-  const bool pair = !small && num_splits == 1;
-  int nt = small ? 1 : NT_PREFILL;
-  auto waves_for = [&](int n) {
-    const long long tiles = ((long long)max_q_len * G + 16 * n - 1) / (16 * n);
-    return pair ? (tiles + 1) / 2 : tiles;
-  };
-  if (nt > 2 && waves_for(nt) * Hk * B < WAVES_TO_FILL) nt = 2;
-  const int waves = (int)waves_for(nt);
-  dim3 grid((waves + 3) / 4, Hk, B * num_splits), block(256);
   const float scale_log2e = scale * 1.4426950408889634f;
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
   }
-#define GO(NT, PM, PAIR)                                                                               \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<NT, PM, PAIR>), grid, block, 0, stream,              \
+  if (small) {
+    // single decoded tokens (at most 16 rows per KV head): one wave per (segment, KV head, split)
+    dim3 grid(1, Hk, B * num_splits), block(256);
+    const int pm = page_shift >= 5 ? 2 : (page_shift >= 3 ? 1 : 0);
+#define GO(PM)                                                                                         \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<PM>), grid, block, 0, stream,                        \
                      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages,                 \
                      (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
                      page_shift, scale_log2e, window, num_splits, part_o, part_ml)
-  const int pm = page_shift >= 5 ? 2 : (page_shift >= 3 ? 1 : 0);
-#define GO3(NT, PAIR)           \
-  do {                          \
-    if (pm == 2) GO(NT, 2, PAIR);      \
-    else if (pm == 1) GO(NT, 1, PAIR); \
-    else GO(NT, 0, PAIR);              \
-  } while (0)
-  if (small) GO3(1, false);
-  else if (nt == 2 && pair) GO3(2, true);
-  else if (nt == 2) GO3(2, false);
-#if NT_PREFILL > 2
-  else if (pair) GO3(NT_PREFILL, true);
-  else GO3(NT_PREFILL, false);
-#endif
-#undef GO3
+    if (pm == 2) GO(2);
+    else if (pm == 1) GO(1);
+    else GO(0);
 #undef GO
+  } else {
+    // prompt portions: 128 rows per workgroup and two waves along the keys, or 64 rows and four
+    // when no segment has more rows than that.  Without a key split a workgroup takes row groups
+    // w and last - w: under the causal mask the two together are one full context long.
+    const long long rows = (long long)max_q_len * G;
+    const int kw = rows > 64 ? 2 : 4;
+    const long long groups = (rows + 256 / kw - 1) / (256 / kw);
+    const int pair = num_splits == 1;
+    const long long items = pair ? (groups + 1) / 2 : groups;
+    if (items * Hk > 0x7fffffffLL || (long long)Hk * page_size * HD * 2 > 0x7fffffffLL) return SA_ERR_ARG;
+    dim3 grid((unsigned)(items * Hk), B * num_splits);
+    const int pm = page_shift >= 3 ? 1 : 0;
+    int rc;
+#define GO(KW, PM)                                                                                       \
+  rc = launch_prompt<KW, PM>(grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, \
+                             (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
+                             page_shift, scale_log2e, window, num_splits, pair, part_o, part_ml)
+    if (kw == 2 && pm == 1) GO(2, 1);
+    else if (kw == 2) GO(2, 0);
+    else if (pm == 1) GO(4, 1);
+    else GO(4, 0);
+#undef GO
+    if (rc != 0) return rc;
+  }
   SA_LAUNCH_CHECK();
   if (num_splits > 1) {
 #define MERGE(S)                                                                                      \

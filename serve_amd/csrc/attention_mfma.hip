@@ -621,7 +621,8 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
   ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);   // bf16 1.0 throughout
 
   for (int pass = 0; pass < 2; ++pass) {
-    const int group = pass == 0 ? item : ngroups - 1 - item;
+    // paired: group `item`, then its mirror image; alone: the groups with the most keys first
+    const int group = (pass == 0) == (pair != 0) ? item : ngroups - 1 - item;
     if (pass == 1) {
       if (!pair || group <= item) break;
       __syncthreads();                                      // the first group's merge has been read
@@ -966,6 +967,8 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
 
 extern "C" int sa_attention_mfma_head_dim() { return HD; }
 
+constexpr int COMPUTE_UNITS = 256;
+
 // A step whose segments have at most 16 rows each (single decoded tokens) takes the one-wave kernel,
 // any other the prompt kernel.
 extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, const void* k_pages,
@@ -1002,12 +1005,13 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
 #undef GO
   } else {
     // prompt portions: 128 rows per workgroup and two waves along the keys, or 64 rows and four
-    // when no segment has more rows than that.  Without a key split a workgroup takes row groups
-    // w and last - w: under the causal mask the two together are one full context long.
+    // when no segment has more rows than that.  Where that still leaves more workgroups than
+    // compute units, a workgroup takes row groups w and last - w: under the causal mask the two
+    // together are one full context long, so all finish at about the same time.
     const long long rows = (long long)max_q_len * G;
     const int kw = rows > 64 ? 2 : 4;
     const long long groups = (rows + 256 / kw - 1) / (256 / kw);
-    const int pair = num_splits == 1;
+    const int pair = num_splits == 1 && (groups + 1) / 2 * Hk * B >= COMPUTE_UNITS;
     const long long items = pair ? (groups + 1) / 2 : groups;
     if (items * Hk > 0x7fffffffLL || (long long)Hk * page_size * HD * 2 > 0x7fffffffLL) return SA_ERR_ARG;
     dim3 grid((unsigned)(items * Hk), B * num_splits);

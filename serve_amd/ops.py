@@ -359,12 +359,23 @@ def mfma_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_strid
             and page_size % 4 == 0 and q_row_stride % 8 == 0 and q.data_ptr() % 16 == 0)
 
 
-def attention_splits(decode_only: bool, num_segments: int, num_kv_heads: int, max_ctx_len: int) -> int:
-    """Into how many parts the key range of a decode step is cut so that the chip is filled:
-    about 512 waves in all (more cost more in the merge than they gain), and no part shorter than
-    64 keys."""
-    if not decode_only:
-        return 1
+def attention_splits(max_q_len: int, num_segments: int, num_kv_heads: int, max_ctx_len: int,
+                     group_size: int = 1) -> int:
+    """Into how many parts the key range of a launch is cut so that the chip is filled.
+    Single decoded tokens: about 512 waves in all (more cost more in the merge than they gain), and
+    no part shorter than 64 keys.  Prompt portions that are at most a quarter of their context (a
+    long prompt taken in portions): about one workgroup of 128 rows per compute unit, parts of at
+    least 1024 keys; portions that are most of their context are never cut, the causal mask makes
+    their parts too unequal."""
+    if max_q_len > 1:
+        if max_ctx_len < 4 * max_q_len:
+            return 1
+        groups = -(-max_q_len * group_size // 128)
+        workgroups = groups * num_kv_heads * num_segments
+        splits = 1
+        while splits < 8 and workgroups * splits < 256 and max_ctx_len // (splits * 2) >= 1024:
+            splits *= 2
+        return splits
     # both inputs are rounded up to powers of two, so that a step run eagerly and the same step
     # replayed from a graph (padded batch, context bucket) cut the keys alike
     ctx = 256
@@ -465,7 +476,8 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
         Hk = k_pages.shape[1]
         # (first segment, segments, tokens up to their end, longest portion, longest context)
         for s0, n, t_end, max_q, max_ctx in _attention_launches(ctx):
-            splits = attention_splits(max_q == 1, n, Hk, max_ctx)
+            # (the parts of a split key range are indexed by token, from the step's first)
+            splits = attention_splits(max_q, n, Hk, max_ctx, num_heads // Hk) if max_q == 1 or s0 == 0 else 1
             paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
                                  t_end, max_q, num_heads, scale, window, splits, s0, n)
         return out

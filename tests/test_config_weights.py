@@ -208,3 +208,18 @@ def test_config_json_of_a_checkpoint_with_all_its_keys():
     hf["rope_scaling"] = {"type": "linear", "factor": 2.0}
     with pytest.raises(Exception, match="linear"):
         LlamaConfig.from_hf_dict(hf)
+
+
+def test_attention_key_splits_are_chosen_by_the_shape_of_the_launch():
+    """Whole prompts are never cut (the causal mask makes the parts unequal), short portions of long
+    contexts and steps of decoded tokens are, until the chip is filled."""
+    from serve_amd.ops import attention_splits
+    assert attention_splits(2048, 1, 8, 2048, 4) == 1
+    assert attention_splits(1024, 2, 8, 1500, 4) == 1
+    assert attention_splits(512, 1, 8, 4096, 4) == 2
+    assert attention_splits(128, 1, 8, 4096, 4) == 4
+    assert attention_splits(256, 1, 8, 1024, 4) == 1           # parts would be shorter than 1024 keys
+    assert attention_splits(512, 8, 8, 4096, 4) == 1           # enough workgroups already
+    assert attention_splits(1, 8, 8, 4096) == 8
+    assert attention_splits(1, 64, 8, 300) == 1
+    assert attention_splits(1, 1, 8, 100000) == 64

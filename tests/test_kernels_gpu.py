@@ -147,7 +147,8 @@ def test_rope_depends_on_distance_only():
 
 
 # ---------------------------------------------------------------------------------------------
-def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False, kernel="simple", splits=1):
+def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False, kernel="simple", splits=1,
+                   poison=False):
     """segs: list of (ctx_before, q_len).  Builds a paged cache with shuffled pages, runs the
     kernel, and compares with dense softmax attention per segment."""
     from serve_amd import ops
@@ -161,6 +162,9 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     rng.shuffle(pages)
     k_pages = rnd((P, Hk, ps, D), DT[dtype], seed + 1)          # unowned pages hold noise
     v_pages = rnd((P, Hk, D, ps), DT[dtype], seed + 2)
+    if poison:                                                  # or NaN: also the rest of a request's last page
+        k_pages.fill_(float("nan"))
+        v_pages.fill_(float("nan"))
     bt = torch.zeros((B, MP), dtype=torch.int32)
     K = [rnd((c + q, Hk, D), DT[dtype], seed + 10 + i) for i, (c, q) in enumerate(segs)]
     V = [rnd((c + q, Hk, D), DT[dtype], seed + 20 + i) for i, (c, q) in enumerate(segs)]
@@ -370,6 +374,31 @@ def test_paged_attention_mfma_ignores_what_lies_beyond_the_context():
             s = torch.einsum("hd,khd->hk", q.double().view(Hq, D), K.double().repeat_interleave(2, 1)) * D ** -0.5
             want = torch.einsum("hk,khd->hd", torch.softmax(s, -1), V.double().repeat_interleave(2, 1)).reshape(1, -1)
             torch.testing.assert_close(out.double(), want, **tol("bfloat16"))
+
+
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 64, 16), (4, 4, 128, 16), (6, 2, 48, 12), (2, 2, 16, 64), (8, 2, 64, 8)])
+def test_prompt_attention_ignores_what_lies_beyond_the_context(Hq, Hk, D, ps):
+    """The same for prompt portions, whose workgroups fetch whole stages of 64 to 256 keys: contexts
+    that end just before, at and just after a stage's edge, few rows and many."""
+    segs = [(0, 37), (100, 28), (0, 129), (250, 7), (0, 200), (127, 1), (0, 256), (3, 125)]
+    attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=500 + D, kernel="mfma", poison=True)
+    attention_case("bfloat16", Hq, Hk, D, ps, [(250, 7), (120, 9), (0, 3)], seed=501 + D, kernel="mfma", poison=True)
+
+
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(8, 2, 64, 16), (4, 1, 128, 32), (3, 3, 80, 20)])
+def test_prompt_attention_long_prompts_windows_and_split_keys(Hq, Hk, D, ps):
+    """Many row groups per segment (a workgroup takes group w and group last - w; an odd count leaves
+    the middle one alone), a window that lets whole stages at the front go unread, and prompt
+    portions over a key range that is split across workgroups."""
+    attention_case("bfloat16", Hq, Hk, D, ps, [(0, 1000), (300, 333)], seed=510 + D, kernel="mfma")
+    attention_case("bfloat16", Hq, Hk, D, ps, [(0, 600), (500, 70)], seed=511 + D, kernel="mfma", window=100)
+    attention_case("bfloat16", Hq, Hk, D, ps, [(900, 40), (2000, 64), (0, 5)], seed=512 + D, kernel="mfma", splits=3,
+                   poison=True)
+    attention_case("bfloat16", Hq, Hk, D, ps, [(700, 20)], seed=513 + D, kernel="mfma", splits=4, window=300)
+    # the way the attention part calls it: a short portion of a long context has its keys split
+    from serve_amd import ops
+    assert ops.attention_splits(200, 1, Hk, 3300, Hq // Hk) > 1
+    attention_case("bfloat16", Hq, Hk, D, ps, [(3100, 200)], seed=514 + D, kernel="dispatch", splits=1)
 
 
 @pytest.mark.parametrize("c_dt", ["bfloat16", "float32"])

@@ -243,27 +243,37 @@ __global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict
 }
 
 // The same for bf16 with (j, j + D/2) pairs over the whole head (rot_dim == D, D % 16 == 0), 16-byte
-// vectors: a thread takes eight pairs of one head (two loads, two stores), then eight dims of one
-// V head (one load, eight scattered stores into the transposed page).
-__global__ __launch_bounds__(256) void rope_kv_write_bf16_vec_kernel(
+// vectors, eight consecutive tokens per block.  A thread takes eight pairs of one head of one token
+// (two loads, two stores).  The values go through LDS: they are read as rows of tokens and written
+// so that neighbouring lanes hold neighbouring tokens of one dim, which in the transposed page
+// ([Hk, D, page_size]) are neighbouring addresses when the tokens' slots are (a prompt portion's
+// are): the two-byte stores of eight lanes then fill one 16-byte run instead of eight memory lines.
+constexpr int ROPE_TOKENS = 8;
+__global__ __launch_bounds__(1024) void rope_kv_write_bf16_vec_kernel(
     bf16_t* __restrict__ qkv, const int* __restrict__ positions, const float* __restrict__ inv_freq,
-    const int* __restrict__ slot, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int Hq, int Hk,
+    const int* __restrict__ slot, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int T, int Hq, int Hk,
     int D, int page_size, int write_kv) {
-  const int t = blockIdx.x;
-  bf16_t* row = qkv + (size_t)t * (size_t)(Hq + (write_kv ? 2 * Hk : 0)) * D;
-  const float pos = (float)positions[t];
-  const int s = write_kv ? slot[t] : -1;
-  const int page = s >= 0 ? s / page_size : 0;
-  const int off = s >= 0 ? s - page * page_size : 0;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rope_lds[];
+  const int t0 = blockIdx.x * ROPE_TOKENS;
+  const int nt = min(ROPE_TOKENS, T - t0);
+  const size_t row_len = (size_t)(Hq + (write_kv ? 2 * Hk : 0)) * D;
   const int half = D >> 1;
   const int gph = half >> 3;                                  // groups of eight pairs per head
   const int Hr = Hq + (write_kv ? Hk : 0);
-  for (int idx = threadIdx.x; idx < Hr * gph; idx += blockDim.x) {
-    const int h = idx / gph;
-    const int j0 = (idx - h * gph) * 8;
-    bf16_t* hp = row + (size_t)h * D;
+  const int per_token = Hr * gph;
+  for (int idx = threadIdx.x; idx < nt * per_token; idx += blockDim.x) {
+    const int i = idx / per_token;
+    const int rem = idx - i * per_token;
+    const int h = rem / gph;
+    const int j0 = (rem - h * gph) * 8;
+    const int t = t0 + i;
+    const float pos = (float)positions[t];
+    bf16_t* hp = qkv + (size_t)t * row_len + (size_t)h * D;
     const uint4 lo = *reinterpret_cast<const uint4*>(hp + j0);
     const uint4 hi = *reinterpret_cast<const uint4*>(hp + half + j0);
+    const float4 f0 = *reinterpret_cast<const float4*>(inv_freq + j0);
+    const float4 f1 = *reinterpret_cast<const float4*>(inv_freq + j0 + 4);
+    const float fr[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
     const uint32_t lw[4] = {lo.x, lo.y, lo.z, lo.w}, hw[4] = {hi.x, hi.y, hi.z, hi.w};
     uint32_t ol[4], oh[4];
 #pragma unroll
@@ -274,7 +284,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16_vec_kernel(
         const float a = bf16_bits_to_float(e ? lw[k] >> 16 : lw[k] & 0xffffu);
         const float b = bf16_bits_to_float(e ? hw[k] >> 16 : hw[k] & 0xffffu);
         float sn, cs;
-        sincos_reduced(pos * inv_freq[j0 + 2 * k + e], &sn, &cs);
+        sincos_reduced(pos * fr[2 * k + e], &sn, &cs);
         o0[e] = a * cs - b * sn;
         o1[e] = b * cs + a * sn;
       }
@@ -283,26 +293,35 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16_vec_kernel(
     }
     bf16_t* dst = hp;
     if (h >= Hq) {
+      const int s = slot[t];
       if (s < 0) continue;
-      dst = k_pages + (((size_t)page * Hk + (h - Hq)) * page_size + off) * D;
+      const int page = s / page_size;
+      dst = k_pages + (((size_t)page * Hk + (h - Hq)) * page_size + (s - page * page_size)) * D;
     }
     *reinterpret_cast<uint4*>(dst + j0) = make_uint4(ol[0], ol[1], ol[2], ol[3]);
     *reinterpret_cast<uint4*>(dst + half + j0) = make_uint4(oh[0], oh[1], oh[2], oh[3]);
   }
-  if (s < 0) return;
-  const int gpv = D >> 3;                                     // groups of eight dims per V head
-  for (int idx = threadIdx.x; idx < Hk * gpv; idx += blockDim.x) {
-    const int h = idx / gpv;
-    const int i0 = (idx - h * gpv) * 8;
-    const uint4 v = *reinterpret_cast<const uint4*>(row + (size_t)(Hq + Hk + h) * D + i0);
-    const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
-    bf16_t* vp = v_pages + (((size_t)page * Hk + h) * D + i0) * page_size + off;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      vp[(size_t)(2 * k) * page_size].v = (uint16_t)(vw[k] & 0xffffu);
-      vp[(size_t)(2 * k + 1) * page_size].v = (uint16_t)(vw[k] >> 16);
-    }
+  if (!write_kv) return;
+  // values: rows of tokens into LDS (16 bytes of padding per row spread the tokens over the banks) ...
+  const int HD = Hk * D;
+  const int stride = HD + 8;                                  // elements
+  uint16_t* tile = reinterpret_cast<uint16_t*>(rope_lds);
+  const int vecs = HD >> 3;
+  for (int idx = threadIdx.x; idx < nt * vecs; idx += blockDim.x) {
+    const int i = idx / vecs;
+    const int e0 = (idx - i * vecs) * 8;
+    *reinterpret_cast<uint4*>(tile + i * stride + e0) =
+        *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + i) * row_len + (size_t)(Hq + Hk) * D + e0);
   }
+  __syncthreads();
+  // ... and out again with the token as the fastest index
+  const int i = threadIdx.x & (ROPE_TOKENS - 1);
+  const int s = i < nt ? slot[t0 + i] : -1;
+  if (s < 0) return;
+  const int page = s / page_size;
+  bf16_t* vp = v_pages + (size_t)page * HD * page_size + (s - page * page_size);
+  for (int e = threadIdx.x / ROPE_TOKENS; e < HD; e += blockDim.x / ROPE_TOKENS)
+    vp[(size_t)e * page_size].v = tile[i * stride + e];
 }
 
 extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, const float* inv_freq,
@@ -313,10 +332,12 @@ extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, 
   if (Hq <= 0 || Hk < 0 || D <= 0 || rot_dim < 0 || rot_dim > D || (rot_dim & 1) || page_size <= 0)
     return SA_ERR_ARG;
   dim3 grid(T), block(256);
+  const size_t tile_bytes = (size_t)ROPE_TOKENS * ((size_t)Hk * D + 8) * 2;
   if (act_dtype == SA_BF16 && cache_dtype == SA_BF16 && !adjacent && rot_dim == D && (D & 15) == 0 &&
-      ((uintptr_t)qkv & 15) == 0) {
-    hipLaunchKernelGGL(rope_kv_write_bf16_vec_kernel, grid, block, 0, stream, (bf16_t*)qkv, positions, inv_freq,
-                       slot, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size, write_kv);
+      ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)inv_freq & 15) == 0 && tile_bytes <= 65536) {
+    hipLaunchKernelGGL(rope_kv_write_bf16_vec_kernel, dim3((T + ROPE_TOKENS - 1) / ROPE_TOKENS), dim3(1024),
+                       write_kv ? tile_bytes : 0, stream, (bf16_t*)qkv, positions, inv_freq, slot, (bf16_t*)k_pages,
+                       (bf16_t*)v_pages, T, Hq, Hk, D, page_size, write_kv);
     SA_LAUNCH_CHECK();
     return 0;
   }

@@ -243,19 +243,20 @@ __global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict
 }
 
 // The same for bf16 with (j, j + D/2) pairs over the whole head (rot_dim == D, D % 16 == 0), 16-byte
-// vectors, eight consecutive tokens per block.  A thread takes eight pairs of one head of one token
-// (two loads, two stores).  The values go through LDS: they are read as rows of tokens and written
+// vectors, `tpb` (1, 2, 4 or 8) consecutive tokens per block.  A thread takes eight pairs of one head of
+// one token (two loads, two stores).  The values go through LDS: they are read as rows of tokens and written
 // so that neighbouring lanes hold neighbouring tokens of one dim, which in the transposed page
 // ([Hk, D, page_size]) are neighbouring addresses when the tokens' slots are (a prompt portion's
 // are): the two-byte stores of eight lanes then fill one 16-byte run instead of eight memory lines.
-constexpr int ROPE_TOKENS = 8;
+// The kernel is bound by the latency of its loads, so the host picks tokens per block and threads
+// per block for many loads in flight: few tokens per block when the step has few tokens.
 __global__ __launch_bounds__(1024) void rope_kv_write_bf16_vec_kernel(
     bf16_t* __restrict__ qkv, const int* __restrict__ positions, const float* __restrict__ inv_freq,
     const int* __restrict__ slot, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int T, int Hq, int Hk,
-    int D, int page_size, int write_kv) {
+    int D, int page_size, int write_kv, int tpb) {
   extern __shared__ __attribute__((aligned(16))) unsigned char rope_lds[];
-  const int t0 = blockIdx.x * ROPE_TOKENS;
-  const int nt = min(ROPE_TOKENS, T - t0);
+  const int t0 = blockIdx.x * tpb;
+  const int nt = min(tpb, T - t0);
   const size_t row_len = (size_t)(Hq + (write_kv ? 2 * Hk : 0)) * D;
   const int half = D >> 1;
   const int gph = half >> 3;                                  // groups of eight pairs per head
@@ -315,12 +316,12 @@ __global__ __launch_bounds__(1024) void rope_kv_write_bf16_vec_kernel(
   }
   __syncthreads();
   // ... and out again with the token as the fastest index
-  const int i = threadIdx.x & (ROPE_TOKENS - 1);
+  const int i = threadIdx.x & (tpb - 1);
   const int s = i < nt ? slot[t0 + i] : -1;
   if (s < 0) return;
   const int page = s / page_size;
   bf16_t* vp = v_pages + (size_t)page * HD * page_size + (s - page * page_size);
-  for (int e = threadIdx.x / ROPE_TOKENS; e < HD; e += blockDim.x / ROPE_TOKENS)
+  for (int e = threadIdx.x / tpb; e < HD; e += blockDim.x / tpb)
     vp[(size_t)e * page_size].v = tile[i * stride + e];
 }
 
@@ -332,12 +333,15 @@ extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, 
   if (Hq <= 0 || Hk < 0 || D <= 0 || rot_dim < 0 || rot_dim > D || (rot_dim & 1) || page_size <= 0)
     return SA_ERR_ARG;
   dim3 grid(T), block(256);
-  const size_t tile_bytes = (size_t)ROPE_TOKENS * ((size_t)Hk * D + 8) * 2;
+  const int tpb = T >= 1024 ? 8 : (T >= 512 ? 4 : (T >= 256 ? 2 : 1));
+  const size_t tile_bytes = (size_t)tpb * ((size_t)Hk * D + 8) * 2;
   if (act_dtype == SA_BF16 && cache_dtype == SA_BF16 && !adjacent && rot_dim == D && (D & 15) == 0 &&
       ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)inv_freq & 15) == 0 && tile_bytes <= 65536) {
-    hipLaunchKernelGGL(rope_kv_write_bf16_vec_kernel, dim3((T + ROPE_TOKENS - 1) / ROPE_TOKENS), dim3(1024),
+    const long long items = (long long)tpb * (Hq + (write_kv ? Hk : 0)) * (D >> 4);   // eight pairs each
+    const int threads = (int)(items >= 1024 ? 1024 : (items <= 256 ? 256 : (items + 63) / 64 * 64));
+    hipLaunchKernelGGL(rope_kv_write_bf16_vec_kernel, dim3((T + tpb - 1) / tpb), dim3(threads),
                        write_kv ? tile_bytes : 0, stream, (bf16_t*)qkv, positions, inv_freq, slot, (bf16_t*)k_pages,
-                       (bf16_t*)v_pages, T, Hq, Hk, D, page_size, write_kv);
+                       (bf16_t*)v_pages, T, Hq, Hk, D, page_size, write_kv, tpb);
     SA_LAUNCH_CHECK();
     return 0;
   }

@@ -130,6 +130,36 @@ def test_rope_kv_write(dtype, Hq, Hk, D, rot, adjacent, ps):
     assert v_pages.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
 
 
+@pytest.mark.parametrize("T", [300, 600, 1100])
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(32, 8, 64, 16), (6, 2, 128, 16), (5, 5, 48, 12)])
+def test_rope_kv_write_of_many_tokens(T, Hq, Hk, D, ps):
+    """Steps of many tokens take several tokens per block (2, 4, 8 from 256, 512, 1024 tokens on) and
+    write the values through LDS: slots that follow one another (a prompt portion, beginning in the
+    middle of a page) and slots all over the cache."""
+    from serve_amd import ops
+    P = -(-T // ps) + 40
+    qkv = rnd((T, (Hq + 2 * Hk) * D), torch.bfloat16, 16)
+    qkv0 = qkv.clone()
+    pos = (torch.arange(T) + 3949).to(torch.int32).to(DEV)
+    inv_freq = (1.0 / (500000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+    run = T // 2 + 3
+    rest = torch.randperm(P * ps - run - 5, generator=torch.Generator().manual_seed(T))[: T - run] + run + 5
+    slots = torch.cat([torch.arange(run) + 5, rest]).to(torch.int32).to(DEV)
+    k_pages = torch.zeros((P, Hk, ps, D), dtype=torch.bfloat16, device=DEV)
+    v_pages = torch.zeros((P, Hk, D, ps), dtype=torch.bfloat16, device=DEV)
+    ops.rope_kv_write(qkv, pos, inv_freq, slots, k_pages, v_pages, Hq, Hk, D, D, False, ps)
+    x = qkv0.double().view(T, Hq + 2 * Hk, D)
+    t = tol("bfloat16")
+    torch.testing.assert_close(qkv.double().view(T, -1, D)[:, :Hq], rope_ref(x[:, :Hq], pos, inv_freq, D, False), **t)
+    page, off = (slots // ps).long(), (slots % ps).long()
+    torch.testing.assert_close(k_pages.double()[page, :, off, :], rope_ref(x[:, Hq:Hq + Hk], pos, inv_freq, D, False), **t)
+    torch.testing.assert_close(v_pages.double()[page, :, :, off], x[:, Hq + Hk:], atol=0, rtol=0)
+    mask = torch.ones((P, ps), dtype=torch.bool, device=DEV)
+    mask[page, off] = False
+    assert k_pages.permute(0, 2, 1, 3)[mask].abs().max().item() == 0
+    assert v_pages.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
+
+
 def test_rope_depends_on_distance_only():
     """<rope(q, m), rope(k, n)> depends on m - n: shift all positions and compare the scores."""
     from serve_amd import ops

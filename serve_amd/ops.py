@@ -443,10 +443,11 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
 # ---------------------------------------------------------------------------------------------
 
 def _attention_launches(ctx):
-    """How a step's segments go to the matrix-core attention kernel.  Single decoded tokens take
-    16-row tiles and a split key range, prompt portions larger tiles: a step that begins with
-    decoding requests and goes on with prompt portions (the order the scheduler gives) is run as
-    two launches, each with the tiles that suit it.  Computed once per step and kept on `ctx`."""
+    """How a step's segments go to the matrix-core attention kernels.  Single decoded tokens take
+    the one-wave kernel and a split key range, prompt portions the kernel that shares keys and
+    values across a workgroup: a step that begins with decoding requests and goes on with prompt
+    portions (the order the scheduler gives) is run as two launches, one of each kind.  Computed
+    once per step and kept on `ctx`."""
     plan = getattr(ctx, "_attention_launches", None)
     if plan is not None:
         return plan

@@ -406,13 +406,18 @@ def test_paged_attention_mfma_ignores_what_lies_beyond_the_context():
             torch.testing.assert_close(out.double(), want, **tol("bfloat16"))
 
 
-@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 64, 16), (4, 4, 128, 16), (6, 2, 48, 12), (2, 2, 16, 64), (8, 2, 64, 8)])
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 64, 16), (4, 4, 128, 16), (6, 2, 48, 12), (2, 2, 16, 64), (8, 2, 64, 8),
+                                        (4, 2, 112, 16), (2, 1, 96, 4)])
 def test_prompt_attention_ignores_what_lies_beyond_the_context(Hq, Hk, D, ps):
     """The same for prompt portions, whose workgroups fetch whole stages of 64 to 256 keys: contexts
     that end just before, at and just after a stage's edge, few rows and many."""
     segs = [(0, 37), (100, 28), (0, 129), (250, 7), (0, 200), (127, 1), (0, 256), (3, 125)]
     attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=500 + D, kernel="mfma", poison=True)
     attention_case("bfloat16", Hq, Hk, D, ps, [(250, 7), (120, 9), (0, 3)], seed=501 + D, kernel="mfma", poison=True)
+    # no segment with more than 64 rows: 64 rows per workgroup and four waves along the keys
+    q = 64 // (Hq // Hk)
+    attention_case("bfloat16", Hq, Hk, D, ps, [(300, q), (0, q - 3), (1000, q // 2 + 1), (129, 5)], seed=502 + D,
+                   kernel="mfma", poison=True)
 
 
 @pytest.mark.parametrize("Hq,Hk,D,ps", [(8, 2, 64, 16), (4, 1, 128, 32), (3, 3, 80, 20)])

@@ -266,13 +266,16 @@ __device__ __forceinline__ void attention_tile(
       }
 
     if (MASKED) {
-      // keys at or beyond the end of the context hold whatever the page held before: their
-      // probability is 0, and 0 times such a value must stay 0
+      // keys at or beyond the end of the context, and keys before the window (whose pages may have
+      // been given back), hold whatever the page held before: their probability is 0, and 0 times
+      // such a value must stay 0
       const int first = key0 + 8 * g;
       uint32_t keep[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        keep[i] = (first + 2 * i < ctx ? 0x0000ffffu : 0u) | (first + 2 * i + 1 < ctx ? 0xffff0000u : 0u);
+      for (int i = 0; i < 4; ++i) {
+        const int k0 = first + 2 * i, k1 = k0 + 1;
+        keep[i] = (k0 < ctx && k0 >= lo_key ? 0x0000ffffu : 0u) | (k1 < ctx && k1 >= lo_key ? 0xffff0000u : 0u);
+      }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         blk.vf[dt].u.x &= keep[0];
@@ -589,20 +592,24 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
       }
     }
   };
-  // registers -> LDS.  Values of keys at or beyond the end of the context hold whatever the page
-  // held before: their probability is 0, and 0 times such a value must stay 0, so they are zeroed.
+  // registers -> LDS.  Values of keys at or beyond the end of the context, and of keys before the
+  // window of the workgroup's first row (their pages may have been given back), hold whatever the
+  // page held before: their probability is 0, and 0 times such a value must stay 0, so they are zeroed.
+  int lo_visible = 0;                                       // first key any row of the workgroup's group sees
   auto stash = [&](int sb, int stage, const Ring& r) __attribute__((always_inline)) {
     unsigned char* st = smem + stage * S::STAGE;
     const int key0 = sb * S::KEYS;
-    const bool at_end = key0 + S::KEYS > ctx;               // the same for every thread
+    const bool at_edge = key0 + S::KEYS > ctx || key0 < lo_visible;   // the same for every thread
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       u32x4_t v = r.v[i];
-      if (at_end) {
+      if (at_edge) {
         const int first = key0 + v_run[i] * 8;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          v[e] &= (first + 2 * e < ctx ? 0x0000ffffu : 0u) | (first + 2 * e + 1 < ctx ? 0xffff0000u : 0u);
+        for (int e = 0; e < 4; ++e) {
+          const int k0 = first + 2 * e, k1 = k0 + 1;
+          v[e] &= (k0 < ctx && k0 >= lo_visible ? 0x0000ffffu : 0u) | (k1 < ctx && k1 >= lo_visible ? 0xffff0000u : 0u);
+        }
       }
       if (S::CHUNKS % 512 == 0 || fetches[i]) {
         *reinterpret_cast<u32x4_t*>(st + k_lds[i]) = r.k[i];
@@ -631,6 +638,7 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
     const int r0g = group * (32 * TW);
     const int hi_key_g = ctx_before + min(rows_total - 1, r0g + 32 * TW - 1) / G;
     const int lo_key_g = window > 0 ? max(0, ctx_before + r0g / G - window + 1) : 0;
+    lo_visible = lo_key_g;
     const int sb_lo = lo_key_g / S::KEYS;
     const int sb_hi = hi_key_g / S::KEYS;
     const int per = (sb_hi - sb_lo + num_splits) / num_splits;

@@ -188,7 +188,7 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     max_ctx = max(c + q for c, q in segs)
     MP = -(-max_ctx // ps)
     P = B * MP + 3
-    pages = list(range(P))
+    pages = list(range(1 if poison else 0, P))                  # poisoned: page 0 (what a table entry of -1 reads) too
     rng.shuffle(pages)
     k_pages = rnd((P, Hk, ps, D), DT[dtype], seed + 1)          # unowned pages hold noise
     v_pages = rnd((P, Hk, D, ps), DT[dtype], seed + 2)
@@ -209,6 +209,9 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
             p = pages.pop()
             bt[i, j] = p
             lo, hi = j * ps, min((j + 1) * ps, c + ql)
+            if poison and window and hi <= c - window + 1:
+                bt[i, j] = -1                                   # no query of the portion sees it: given back
+                continue
             k_pages[p, :, : hi - lo, :] = K[i][lo:hi].permute(1, 0, 2)
             v_pages[p, :, :, : hi - lo] = V[i][lo:hi].permute(1, 2, 0)
     cu = [0]
@@ -430,6 +433,11 @@ def test_prompt_attention_long_prompts_windows_and_split_keys(Hq, Hk, D, ps):
     attention_case("bfloat16", Hq, Hk, D, ps, [(900, 40), (2000, 64), (0, 5)], seed=512 + D, kernel="mfma", splits=3,
                    poison=True)
     attention_case("bfloat16", Hq, Hk, D, ps, [(700, 20)], seed=513 + D, kernel="mfma", splits=4, window=300)
+    # pages that the window has passed are given back (table entry -1) and hold anything
+    attention_case("bfloat16", Hq, Hk, D, ps, [(0, 600), (500, 70), (433, 1), (90, 2)], seed=515 + D, kernel="mfma",
+                   window=100, poison=True)
+    attention_case("bfloat16", Hq, Hk, D, ps, [(433, 1), (90, 1), (1000, 1)], seed=516 + D, kernel="mfma", window=100,
+                   poison=True, splits=2)
     # the way the attention part calls it: a short portion of a long context has its keys split
     from serve_amd import ops
     assert ops.attention_splits(200, 1, Hk, 3300, Hq // Hk) > 1

@@ -211,3 +211,57 @@ def test_odd_sizes(tmp_path, name, page_size, dtype):
     tokens = util.random_tokens(rng, 90, cfg.vocab_size)
     got = run_portions(engine, "r", tokens, [70, 2, 17, 1])
     util.assert_close(got, util.plain_logits(folder, tokens), dtype, f"{name} page {page_size}")
+
+
+@pytest.mark.parametrize("seed", [3, 5, 7, 9])
+def test_random_configurations_random_cuts(tmp_path, seed):
+    """A configuration drawn at random (head size 16..128, groups 1..5, odd widths, 1..3 layers,
+    scaled rotation or not, tied head or not, page size 4..64) and three requests of up to 700 tokens,
+    cut at random into portions of 1 to 300 tokens and batched in random order with just enough
+    pages: every logit, in both dtypes, against the plain model."""
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.llama import Llama3RopeScaling, LlamaConfig
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    from serve_amd.weights.loader import write_random_model
+    rng = random.Random(seed)
+    kv_heads, group = rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 4, 5])
+    cfg = LlamaConfig(vocab_size=rng.randrange(50, 900), hidden_size=rng.choice([64, 72, 96, 128, 136, 200, 256]),
+                      intermediate_size=8 * rng.randrange(8, 60), num_hidden_layers=rng.choice([1, 2, 3]),
+                      num_attention_heads=kv_heads * group, num_key_value_heads=kv_heads,
+                      head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128]), rms_norm_eps=rng.choice([1e-5, 1e-6]),
+                      rope_theta=rng.choice([10000.0, 500000.0]),
+                      rope_scaling=rng.choice([None, Llama3RopeScaling(8.0, 1.0, 4.0, 64)]),
+                      tie_word_embeddings=rng.choice([True, False]))
+    page_size = rng.choice([4, 8, 12, 16, 32, 64])
+    lengths = [rng.randrange(40, 700) for _ in range(3)]
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=seed)
+    tokens = [util.random_tokens(rng, n, cfg.vocab_size) for n in lengths]
+    want = [util.plain_logits(folder, t) for t in tokens]
+    for dtype in DTYPES:
+        pages = sum(-(-n // page_size) for n in lengths) + 2
+        engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=page_size, num_pages=pages,
+                                                        max_context=1024, max_requests=4, max_tokens_per_step=4096,
+                                                        prefill_chunk=4096))
+        cuts = random.Random(seed * 7 + 1)
+        at, got = [0, 0, 0], [[], [], []]
+        for i in range(3):
+            engine.runner.admit(i)
+        while any(at[i] < lengths[i] for i in range(3)):
+            order = [i for i in range(3) if at[i] < lengths[i] and cuts.random() < 0.8]
+            cuts.shuffle(order)
+            segs = []
+            for i in order:
+                n = min(lengths[i] - at[i], cuts.choice([1, 1, 2, 3, 17, 64, 130, 300]))
+                segs.append(Segment(i, tokens[i][at[i]: at[i] + n], list(range(n))))
+                at[i] += n
+            if not segs:
+                continue
+            out = engine.step(segs)
+            row = 0
+            for s in segs:
+                got[s.req_id].append(out[row: row + len(s.tokens)])
+                row += len(s.tokens)
+        for i in range(3):
+            util.assert_close(torch.cat(got[i]), want[i], dtype, f"seed {seed} request {i} {dtype}: {cfg}, page {page_size}")
+            engine.runner.release(i)

@@ -433,8 +433,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 // What the time goes to is the number of instructions a SIMD has to issue: measured on this chip,
 // a SIMD whose two waves keep the vector unit busy gains little from matrix instructions of the
 // other wave running beside them (288 vector + 32 matrix instructions: 429 ns + 229 ns apart,
-// 589 ns together), and an exponential costs about three and a half ordinary vector instructions.
-// Hence one softmax update per 64 keys, three-way maxima, row sums taken by the matrix cores, O
+// 589 ns together); exponentials, three and a half times as slow as plain vector instructions when
+// alone, do run beside those.  Hence one softmax update per 64 keys, three-way maxima, row sums taken by the matrix cores, O
 // rescaled only when a maximum has moved, and page addresses that are a constant plus a product.
 //
 // The work per stage is the same straight line of code for every wave and stage: a block that is

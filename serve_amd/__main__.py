@@ -18,10 +18,15 @@ import sys
 
 def _generate(argv) -> int:
     ap = argparse.ArgumentParser(prog="python -m serve_amd generate")
-    ap.add_argument("--model", required=True, help="model folder (config.json + model.safetensors)")
+    src = ap.add_mutually_exclusive_group(required=True)
+    src.add_argument("--model", help="model folder (config.json + model.safetensors)")
+    src.add_argument("--shape", help="a named shape with random weights drawn from --seed (tiny, tiny-a, tiny-b, "
+                     "llama-1b, llama-3b, llama-8b)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--prompt-ids", help="file with one prompt a line: JSON list or blank-separated token ids "
                     "(default: standard input)")
+    ap.add_argument("--random-prompts", metavar="N:LEN", help="N prompts of LEN uniform random token ids "
+                    "instead of --prompt-ids")
     ap.add_argument("--max-new-tokens", type=int, default=32)
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy (serve/run.py:56-57)")
     ap.add_argument("--seed", type=int, default=0)
@@ -38,17 +43,32 @@ def _generate(argv) -> int:
 
     from .config.engine import EngineConfig
     from .engine.engine import Engine, Request
-    src = open(args.prompt_ids) if args.prompt_ids else sys.stdin
-    prompts = []
-    for line in src:
-        line = line.strip()
-        if line:
-            prompts.append(json.loads(line) if line.startswith("[") else [int(t) for t in line.split()])
     cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, num_pages=args.num_pages,
                        memory_fraction=args.memory_fraction, max_context=args.max_context,
                        max_requests=args.max_requests, max_tokens_per_step=args.max_tokens_per_step,
                        prefill_chunk=args.prefill_chunk, admission=args.admission, seed=args.seed)
-    engine = Engine.from_folder(args.model, cfg)
+    if args.model:
+        engine = Engine.from_folder(args.model, cfg)
+    else:
+        from .benchmark import SHAPES
+        if args.shape not in SHAPES:
+            ap.error(f"unknown shape {args.shape!r}; known: {sorted(SHAPES)}")
+        engine = Engine.from_config(SHAPES[args.shape], args.seed, cfg)
+    prompts = []
+    if args.random_prompts:
+        import random
+        try:
+            count, length = (int(x) for x in args.random_prompts.split(":"))
+        except ValueError:
+            ap.error("--random-prompts takes N:LEN, for instance 4:128")
+        rng = random.Random(args.seed)
+        vocab = engine.model.spec.vocab_size
+        prompts = [[rng.randrange(vocab) for _ in range(length)] for _ in range(count)]
+    else:
+        for line in (open(args.prompt_ids) if args.prompt_ids else sys.stdin):
+            line = line.strip()
+            if line:
+                prompts.append(json.loads(line) if line.startswith("[") else [int(t) for t in line.split()])
     out = engine.generate([Request(torch.tensor(p, dtype=torch.long), len(p), args.max_new_tokens) for p in prompts],
                           temperature=args.temperature)
     for r in out:
@@ -60,7 +80,7 @@ def _random_model(argv) -> int:
     ap = argparse.ArgumentParser(prog="python -m serve_amd random-model")
     ap.add_argument("--out", required=True, help="folder to write config.json and model.safetensors into")
     g = ap.add_mutually_exclusive_group(required=True)
-    g.add_argument("--shape", help="a named shape (tiny, llama-1b, llama-3b, llama-8b)")
+    g.add_argument("--shape", help="a named shape (tiny, tiny-a, tiny-b, llama-1b, llama-3b, llama-8b)")
     g.add_argument("--config", help="a config.json to take the sizes from")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args(argv)

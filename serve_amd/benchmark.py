@@ -28,6 +28,14 @@ _L3 = lambda factor: Llama3RopeScaling(factor, 1.0, 4.0, 8192)   # noqa: E731
 SHAPES = {
     "tiny": LlamaConfig(vocab_size=10000, hidden_size=64, intermediate_size=192, num_hidden_layers=2,
                         num_attention_heads=4, num_key_value_heads=2, head_dim=16),
+    # the two tiny configurations that the engine's equality checks are specified on
+    "tiny-a": LlamaConfig(vocab_size=256, hidden_size=64, intermediate_size=192, num_hidden_layers=2,
+                          num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-5,
+                          rope_theta=10000.0, tie_word_embeddings=False),
+    "tiny-b": LlamaConfig(vocab_size=512, hidden_size=96, intermediate_size=256, num_hidden_layers=3,
+                          num_attention_heads=3, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-6,
+                          rope_theta=500000.0, rope_scaling=Llama3RopeScaling(32.0, 1.0, 4.0, 64),
+                          tie_word_embeddings=True),
     "llama-1b": LlamaConfig(vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_hidden_layers=16,
                             num_attention_heads=32, num_key_value_heads=8, head_dim=64, rope_theta=500000.0,
                             rope_scaling=_L3(32.0), tie_word_embeddings=True),

@@ -84,10 +84,16 @@ class Engine:
         return self.runner.step(segments)
 
     def generate(self, requests: Sequence[Request], temperature: Union[float, Sequence[float]] = 0.0,
-                 return_logits: bool = False) -> List[Request]:
+                 return_logits: Union[bool, str] = False) -> List[Request]:
         """Generate `max_new_tokens` tokens for every request; results in the order given
         (serve/run.py:304).  `temperature` 0 is greedy (serve/run.py:56-57); one value for all
-        requests as in the reference, or one per request."""
+        requests as in the reference, or one per request.  `return_logits`: False / "none"; True /
+        "last": the fp32 logits [V] that the last token was drawn from, as the reference returns
+        them (serve/run.py:229-230); "all": those of every generated token, [generated, V]."""
+        if return_logits not in (False, True, "none", "last", "all"):
+            raise ValueError(f"return_logits must be False, True, 'none', 'last' or 'all', not {return_logits!r}")
+        keep_all = return_logits == "all"
+        keep_last = return_logits is True or return_logits == "last"
         temps = list(temperature) if isinstance(temperature, (list, tuple)) else [float(temperature)] * len(requests)
         if len(temps) != len(requests):
             raise ValueError("one temperature per request is needed")
@@ -97,7 +103,7 @@ class Engine:
             if r.input_length != len(ids):
                 raise ValueError(f"request {i}: input_length {r.input_length} != len(input_ids) {len(ids)}")
             gen.append(GenerationRequest(req_id=i, prompt=ids, max_new_tokens=int(r.max_new_tokens),
-                                         temperature=float(t), keep_logits=return_logits))
+                                         temperature=float(t), keep_logits=keep_last, keep_all_logits=keep_all))
         sched = Scheduler(self.runner, self.sampler, self.cfg, eos_token_ids=None)
         done = sched.run(gen)
         out = []
@@ -105,7 +111,8 @@ class Engine:
             out.append(Request(input_ids=r.input_ids, input_length=r.input_length,
                                max_new_tokens=r.max_new_tokens,
                                generated_tokens=torch.tensor(g.generated, dtype=torch.long),
-                               logits=g.last_logits if return_logits else None))
+                               logits=(torch.stack(g.logit_rows) if keep_all and g.logit_rows
+                                       else g.last_logits if keep_last else None)))
         return out
 
 
@@ -122,6 +129,6 @@ def load_model(model_name: str, device: str = "cuda", dtype=torch.bfloat16, **en
 
 
 def generate(model: Engine, requests: Sequence[Request], temperature: float = 0.0,
-             return_logits: bool = False) -> List[Request]:
+             return_logits: Union[bool, str] = False) -> List[Request]:
     """serve/run.py:238-308."""
     return model.generate(requests, temperature=temperature, return_logits=return_logits)

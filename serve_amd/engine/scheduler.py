@@ -35,10 +35,12 @@ class GenerationRequest:
     prompt: List[int]
     max_new_tokens: int
     temperature: float = 0.0
-    keep_logits: bool = False
+    keep_logits: bool = False            # keep the logits the last token was drawn from (serve/run.py:229-230)
+    keep_all_logits: bool = False        # ... those of every generated token, in `logit_rows`
     # results
     generated: List[int] = field(default_factory=list)
     last_logits: object = None
+    logit_rows: List[object] = field(default_factory=list)
     error: Optional[str] = None
     preemptions: int = 0
     # progress: tokens of prompt + generated that are in the cache
@@ -280,6 +282,8 @@ class Scheduler:
             r.fed += n
         for i, (r, tok) in enumerate(zip(samplers, tokens)):
             r.generated.append(int(tok))
+            if r.keep_all_logits:
+                r.logit_rows.append(logits[i].clone())
             if r.done() or int(tok) in self.eos:
                 if r.keep_logits:
                     r.last_logits = logits[i].clone()
@@ -296,7 +300,7 @@ class Scheduler:
         None: the host needs the tokens first."""
         if not self.async_decode:
             return None
-        if any(r.keep_logits for r in plan.requests):
+        if any(r.keep_logits or r.keep_all_logits for r in plan.requests):
             return None
         if self._inflight is not None:
             before = {id(r) for r in self._inflight[1]}

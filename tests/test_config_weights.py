@@ -223,3 +223,23 @@ def test_attention_key_splits_are_chosen_by_the_shape_of_the_launch():
     assert attention_splits(1, 8, 8, 4096) == 8
     assert attention_splits(1, 64, 8, 300) == 1
     assert attention_splits(1, 1, 8, 100000) == 64
+
+
+def test_named_shapes_are_the_configurations_the_measurements_are_specified_on():
+    """`--shape tiny-a | tiny-b | llama-1b | llama-3b | llama-8b`: every size the specification of the
+    benchmark configurations gives (BASELINE.json, read as text: it is prose) appears in the preset."""
+    from serve_amd.benchmark import SHAPES
+    a, b, one = SHAPES["tiny-a"], SHAPES["tiny-b"], SHAPES["llama-1b"]
+    assert (a.num_hidden_layers, a.hidden_size, a.num_attention_heads, a.num_key_value_heads, a.head_dim,
+            a.intermediate_size, a.vocab_size, a.rope_theta, a.rope_scaling, a.rms_norm_eps, a.tie_word_embeddings) == \
+        (2, 64, 4, 2, 16, 192, 256, 10000.0, None, 1e-5, False)
+    assert (b.num_hidden_layers, b.hidden_size, b.num_attention_heads, b.num_key_value_heads, b.head_dim,
+            b.intermediate_size, b.vocab_size, b.rope_theta, b.rms_norm_eps, b.tie_word_embeddings) == \
+        (3, 96, 3, 1, 32, 256, 512, 500000.0, 1e-6, True)
+    s = b.rope_scaling
+    assert (s.factor, s.low_freq_factor, s.high_freq_factor, s.original_max_position_embeddings) == (32.0, 1.0, 4.0, 64)
+    assert (one.num_hidden_layers, one.hidden_size, one.num_attention_heads, one.num_key_value_heads, one.head_dim,
+            one.intermediate_size, one.vocab_size, one.tie_word_embeddings) == (16, 2048, 32, 8, 64, 8192, 128256, True)
+    assert SHAPES["llama-3b"].num_hidden_layers == 28 and SHAPES["llama-8b"].intermediate_size == 14336
+    for cfg in SHAPES.values():
+        cfg.validate()

@@ -78,6 +78,46 @@ def test_sampled_generation_tiny_b_chunked_beside_decodes(tmp_path, dtype):
         assert alone[0].generated_tokens.tolist() == out[0].generated_tokens.tolist()
 
 
+def test_logits_of_the_last_or_of_every_generated_token(tmp_path):
+    """`return_logits`: True / "last" as the reference (the logits the last token came from), "all"
+    those of every generated token; each row is the plain model's logits at that place."""
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine, Request
+    folder = util.make_folder(tmp_path, "A")
+    eng = Engine.from_folder(folder, EngineConfig(dtype="float32", page_size=4, num_pages=32, max_context=64,
+                                                 max_requests=4, prefill_chunk=8, max_tokens_per_step=10))
+    rng = random.Random(5)
+    prompts = [util.random_tokens(rng, n, 256) for n in (7, 13, 1)]
+    reqs = [Request(torch.tensor(p), len(p), 5) for p in prompts]
+    every = eng.generate(reqs, temperature=0.0, return_logits="all")
+    last = eng.generate(reqs, temperature=0.0, return_logits=True)
+    none = eng.generate(reqs, temperature=0.0)
+    for p, a, b, c in zip(prompts, every, last, none):
+        toks = a.generated_tokens.tolist()
+        assert toks == b.generated_tokens.tolist() == c.generated_tokens.tolist() and c.logits is None
+        assert tuple(a.logits.shape) == (5, 256) and tuple(b.logits.shape) == (256,)
+        assert a.logits.argmax(-1).tolist() == toks
+        torch.testing.assert_close(a.logits[-1], b.logits, atol=0, rtol=0)
+        want = util.plain_logits(folder, p + toks[:-1])[len(p) - 1:]
+        util.assert_close(a.logits, want, "float32", "logits of every generated token")
+    with pytest.raises(ValueError, match="return_logits"):
+        eng.generate(reqs, return_logits="some")
+
+
+def test_command_line_generates_from_a_named_shape(tmp_path):
+    """`python -m serve_amd generate --shape tiny-a --random-prompts 2:9`: random weights and random
+    prompts from the seed, one JSON list of generated ids a line; the same call gives the same ids."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, "-m", "serve_amd", "generate", "--shape", "tiny-a", "--random-prompts", "2:9",
+           "--max-new-tokens", "4", "--dtype", "float32", "--num-pages", "16", "--page-size", "4", "--max-context", "32",
+           "--max-requests", "4", "--seed", "3"]
+    runs = [subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=300) for _ in range(2)]
+    for r in runs:
+        assert r.returncode == 0, r.stderr[-2000:]
+    lines = [[json.loads(l) for l in r.stdout.splitlines() if l.startswith("[")] for r in runs]
+    assert lines[0] == lines[1] and len(lines[0]) == 2 and all(len(x) == 4 for x in lines[0])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_few_pages_preemption_gives_the_same_tokens(tmp_path, dtype):
     from serve_amd.config.engine import EngineConfig

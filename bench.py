@@ -111,6 +111,59 @@ def prefill_run(engine, tokens: int, repeats: int, seed: int):
     return best
 
 
+def measured_ceilings():
+    """What the device itself reaches with the library's plain operations: a copy of 1 GiB (bytes
+    read + written per second), a reduction over 1 GiB (bytes read per second), and a square bf16
+    product of 8192 (flops per second)."""
+    import torch
+    dev = "cuda:0"
+
+    def best(fn, repeats=5):
+        times = []
+        for _ in range(repeats + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        return min(times[1:])
+
+    n = 512 * 1024 * 1024
+    src = torch.ones(n, dtype=torch.bfloat16, device=dev)
+    dst = torch.empty_like(src)
+    copy = 2 * 2 * n / best(lambda: dst.copy_(src))
+    read = 2 * n / best(lambda: torch.sum(src, dtype=torch.float32))
+    del src, dst
+    a = torch.randn(8192, 8192, dtype=torch.bfloat16, device=dev)
+    b = torch.randn(8192, 8192, dtype=torch.bfloat16, device=dev)
+    c = torch.empty(8192, 8192, dtype=torch.bfloat16, device=dev)
+    gemm = 2 * 8192 ** 3 / best(lambda: torch.mm(a, b.t(), out=c))
+    return {"copy": copy, "read": read, "gemm": gemm}
+
+
+def report(engine, cfg, steps: int, warmup: int) -> int:
+    """`--report`: every number of the measurement with the bytes or flops it stands for, as a
+    share of the published peaks and of the ceilings measured on this device."""
+    ceil = measured_ceilings()
+    print(f"measured ceilings: copy {ceil['copy'] / 1e12:.2f} TB/s (read + write), reduction "
+          f"{ceil['read'] / 1e12:.2f} TB/s (read), 8192^3 bf16 product {ceil['gemm'] / 1e15:.3f} PFLOP/s")
+    bw = max(ceil["copy"], ceil["read"])
+    print(f"{'workload':34s} {'ms/step':>8s} {'tokens/s':>10s} {'GB or TFLOP':>12s} {'achieved':>14s} {'of peak':>8s} "
+          f"{'of measured':>11s}")
+    for batch, prompt_len, n in ((1, 256, 250), (8, 256, 250), (64, 256, 250), (8, 4096 - steps - warmup - 3, steps)):
+        dt, mean_ctx = decode_run(engine, batch, prompt_len, warmup if prompt_len > 256 else 4, n, seed=20 + batch)
+        nbytes = weight_bytes(cfg) + batch * mean_ctx * kv_bytes_per_token(cfg)
+        rate = nbytes / (dt / n)
+        print(f"{f'decode, batch {batch}, context ~{int(mean_ctx)}':34s} {dt / n * 1e3:8.3f} {batch * n / dt:10.0f} "
+              f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}")
+    T = 2048
+    pt = prefill_run(engine, T, repeats=5, seed=7)
+    fl = prefill_flops(cfg, T)
+    print(f"{'prefill, 2,048 tokens':34s} {pt * 1e3:8.3f} {T / pt:10.0f} {fl / 1e12:6.3f} TFLOP {fl / pt / 1e15:7.3f} PFLOP/s "
+          f"{fl / pt / BF16_PEAK:8.3f} {fl / pt / ceil['gemm']:11.3f}")
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -124,6 +177,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch-1/64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own short JSON line")
+    ap.add_argument("--report", action="store_true",
+                    help="print a table instead of the JSON line: decode at batch 1, 8 and 64 and the prefill, each "
+                    "with its bytes or flops, as a share of the published peaks and of ceilings measured here")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -150,6 +206,8 @@ def main() -> int:
         print(json.dumps({"prefill": {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
                                       "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}}), flush=True)
         return 0
+    if args.report:
+        return report(engine, cfg, args.steps, args.warmup)
     steps, warmup = args.steps, args.warmup
     prompt_len = args.context - (warmup + steps + 3)
     if prompt_len < 1:
@@ -183,7 +241,7 @@ def main() -> int:
         out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
                           "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}
         points = {}
-        for b in (1, 64):
+        for b in (1, 8, 64):
             d, _ = decode_run(engine, b, 256, 4, 250, seed=10 + b)
             points[f"decode_b{b}"] = round(b * 250 / d, 1)
         out["points"] = points

@@ -423,6 +423,19 @@ def test_prompt_attention_ignores_what_lies_beyond_the_context(Hq, Hk, D, ps):
                    kernel="mfma", poison=True)
 
 
+@pytest.mark.parametrize("Hq,Hk,D,ps,segs", [
+    (32, 8, 64, 16, [(0, 512), (100, 530), (0, 512), (37, 600)]),
+    (16, 8, 128, 16, [(0, 1100), (3, 1030), (0, 1024), (500, 1111)]),
+    (40, 8, 48, 12, [(0, 300), (0, 410), (77, 260), (0, 415), (5, 401)])])
+def test_prompt_attention_with_row_groups_in_pairs(Hq, Hk, D, ps, segs):
+    """With at least as many workgroups as compute units left after pairing, a workgroup takes row
+    group w of its segment and then group last - w (segments with even and odd numbers of groups,
+    and fewer groups than the longest segment has)."""
+    groups = -(-max(q for _, q in segs) * (Hq // Hk) // 128)
+    assert (groups + 1) // 2 * Hk * len(segs) >= 256, "the case would not be paired"
+    attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=520 + D, kernel="mfma", poison=True)
+
+
 @pytest.mark.parametrize("Hq,Hk,D,ps", [(8, 2, 64, 16), (4, 1, 128, 32), (3, 3, 80, 20)])
 def test_prompt_attention_long_prompts_windows_and_split_keys(Hq, Hk, D, ps):
     """Many row groups per segment (a workgroup takes group w and group last - w; an odd count leaves

@@ -333,7 +333,8 @@ extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, 
   if (Hq <= 0 || Hk < 0 || D <= 0 || rot_dim < 0 || rot_dim > D || (rot_dim & 1) || page_size <= 0)
     return SA_ERR_ARG;
   dim3 grid(T), block(256);
-  const int tpb = T >= 1024 ? 8 : (T >= 512 ? 4 : (T >= 256 ? 2 : 1));
+  int tpb = T >= 1024 ? 8 : (T >= 512 ? 4 : (T >= 256 ? 2 : 1));
+  while (tpb > 1 && (size_t)tpb * ((size_t)Hk * D + 8) * 2 > 65536) tpb >>= 1;   // the values' tile has to fit LDS
   const size_t tile_bytes = (size_t)tpb * ((size_t)Hk * D + 8) * 2;
   if (act_dtype == SA_BF16 && cache_dtype == SA_BF16 && !adjacent && rot_dim == D && (D & 15) == 0 &&
       ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)inv_freq & 15) == 0 && tile_bytes <= 65536) {

@@ -131,7 +131,7 @@ def test_rope_kv_write(dtype, Hq, Hk, D, rot, adjacent, ps):
 
 
 @pytest.mark.parametrize("T", [300, 600, 1100])
-@pytest.mark.parametrize("Hq,Hk,D,ps", [(32, 8, 64, 16), (6, 2, 128, 16), (5, 5, 48, 12)])
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(32, 8, 64, 16), (6, 2, 128, 16), (5, 5, 48, 12), (36, 36, 128, 16)])
 def test_rope_kv_write_of_many_tokens(T, Hq, Hk, D, ps):
     """Steps of many tokens take several tokens per block (2, 4, 8 from 256, 512, 1024 tokens on) and
     write the values through LDS: slots that follow one another (a prompt portion, beginning in the
@@ -410,7 +410,7 @@ def test_paged_attention_mfma_ignores_what_lies_beyond_the_context():
 
 
 @pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 64, 16), (4, 4, 128, 16), (6, 2, 48, 12), (2, 2, 16, 64), (8, 2, 64, 8),
-                                        (4, 2, 112, 16), (2, 1, 96, 4)])
+                                        (4, 2, 112, 16), (2, 1, 96, 4), (4, 2, 64, 256), (2, 1, 128, 512)])
 def test_prompt_attention_ignores_what_lies_beyond_the_context(Hq, Hk, D, ps):
     """The same for prompt portions, whose workgroups fetch whole stages of 64 to 256 keys: contexts
     that end just before, at and just after a stage's edge, few rows and many."""

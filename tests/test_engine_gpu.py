@@ -265,3 +265,36 @@ def test_random_configurations_random_cuts(tmp_path, seed):
         for i in range(3):
             util.assert_close(torch.cat(got[i]), want[i], dtype, f"seed {seed} request {i} {dtype}: {cfg}, page {page_size}")
             engine.runner.release(i)
+
+
+def test_llama_1b_layer_sizes(tmp_path):
+    """The widths of Llama-3.2-1B (hidden 2048, 32 heads in 8 groups of head size 64, feed-forward
+    8192, vocabulary 128256, tied head, scaled rotation) with two layers: products cut along K, the
+    head over the whole vocabulary and attention with four query heads per KV head at the sizes the
+    measurements run at, which the tiny configurations cannot show.  float32 within the float32
+    tolerance of the plain model.  bfloat16 rounds every activation to 8 bits: at this width the
+    2e-2 that holds for the tiny models does not, so the bound is stated in units of the logits'
+    spread: mean error at most 1 % of their standard deviation, no logit off by more than 6 %."""
+    import dataclasses
+
+    from serve_amd.benchmark import SHAPES
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine
+    from serve_amd.weights.loader import write_random_model
+    cfg = dataclasses.replace(SHAPES["llama-1b"], num_hidden_layers=2)
+    folder = write_random_model(str(tmp_path / "wide"), cfg, seed=0)
+    tokens = util.random_tokens(random.Random(0), 48, cfg.vocab_size)
+    want = util.plain_logits(folder, tokens)
+    for dtype in DTYPES:
+        engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=16, num_pages=16, max_context=128,
+                                                        max_requests=2))
+        got = run_portions(engine, "r", tokens, [29, 2, 16, 1]).double().cpu()
+        if dtype == "float32":
+            util.assert_close(got, want, dtype, "1B layer sizes")
+        else:
+            err, spread = (got - want).abs(), want.std().item()
+            assert err.mean().item() <= 0.01 * spread and err.max().item() <= 0.06 * spread, \
+                f"bfloat16 at 1B layer sizes: mean error {err.mean().item():.4f}, max {err.max().item():.4f}, " \
+                f"spread of the logits {spread:.3f}"
+        del engine
+        torch.cuda.empty_cache()

@@ -43,11 +43,14 @@ def _dev(*tensors: Optional[torch.Tensor]) -> None:
     for t in tensors:
         if t is None:
             continue
-        _check(t.is_cuda, "serve_amd kernels run on the GPU only; got a tensor on " + str(t.device))
-        _check(t.is_contiguous(), "kernel arguments must be contiguous")
+        if not t.is_cuda:
+            raise KernelError("serve_amd kernels run on the GPU only; got a tensor on " + str(t.device))
+        if not t.is_contiguous():
+            raise KernelError("kernel arguments must be contiguous")
         if dev is None:
             dev = t.device
-        _check(t.device == dev, "kernel arguments lie on different devices")
+        elif t.device != dev:
+            raise KernelError("kernel arguments lie on different devices")
 
 
 def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
@@ -55,7 +58,9 @@ def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
 
 
 def _stream() -> c_void_p:
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the current stream of the current device as a raw handle (what torch.cuda.current_stream()
+    # wraps into an object, at thirty times the cost: this runs once per kernel launch)
+    return c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def _ret(code: int, what: str) -> None:

@@ -1,6 +1,6 @@
 // bf16 matrix products on the matrix cores for few rows of activations (decode steps and short
 // prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
-// Two kernels: gemm_skinny_kernel for up to 16 rows, gemm_mid_kernel for 17 to 64 (per pass).
+// Two kernels: gemm_skinny_kernel for one or two rows, gemm_mid_kernel for up to 64 (per pass).
 //
 // The work is bound by reading W.  In the first, a wave owns RT tiles of 16 rows of W and walks a
 // slice of K in steps of 32; the KS waves of a workgroup split K between them and add their partial sums
@@ -301,8 +301,8 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, ql, g, c);
 }
 
-// The same products for 17..64 rows of activations (decode at larger batches, short prompt
-// portions).  With that many rows a workgroup reads about as many bytes of activations as of
+// The same products for up to 64 rows of activations (decode at all but the smallest batches, short
+// prompt portions).  With that many rows a workgroup reads about as many bytes of activations as of
 // weights, so the activations are staged through LDS and shared.  A workgroup has NR x KH waves:
 // NR groups of weight rows times KH slices of each 256-wide stage of K; the NR waves of a slice read
 // the same activation fragments, and the KH slices add their sums through LDS at the end, in order.
@@ -512,28 +512,49 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
   return 0;
 }
 
+// up to this many rows take gemm_skinny_kernel, more take gemm_mid_kernel
+// Which kernel and which workgroup shape a product takes, from a sweep over both kernels and their
+// shapes at the sizes of the Llama-3 family (widths 2048 to 4096), 1 to 64 rows, weights cold.
+// gemm_skinny_kernel, where every wave fetches its own activation rows, wins only at one or two rows
+// (and for the small fused q/k/v products up to eight); from there on sharing the activations of a
+// workgroup through LDS is faster, and the question is how many weight rows a workgroup takes
+// (more halve the activation traffic, fewer give more workgroups) and how many ways it cuts a stage
+// of K.  Few weight rows in all: small workgroups, K cut often; many: 128 rows a workgroup.
+template <typename TC, int EPI>
+static bool takes_skinny(int M, int N, const QkvRopeArgs& qa) {
+  if (EPI == EPI_QKV_ROPE) return (qa.Hq + 2 * qa.Hk) * (qa.D >> 4) < 256 && M <= 8;
+  return M <= 2;
+}
+
 template <typename TC, int EPI>
 static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                     const QkvRopeArgs& qa, hipStream_t stream) {
-  const bool four = M > 32;
+  const int mt = M > 32 ? 4 : (M > 16 ? 2 : 1);      // 16-row tiles of activations per pass
 #define GO(RT, MT, NR, KH) \
   return launch_mid<RT, MT, NR, KH, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
+#define GO3(RT, NR1, KH1, NR2, KH2, NR4, KH4) \
+  do {                                         \
+    if (mt == 1) GO(RT, 1, NR1, KH1);          \
+    if (mt == 2) GO(RT, 2, NR2, KH2);          \
+    GO(RT, 4, NR4, KH4);                       \
+  } while (0)
   if constexpr (EPI == EPI_PLAIN) {
-    if (N < 8192) {                  // few weight rows: 32 a workgroup, K cut four ways inside it
-      if (four) GO(1, 4, 2, 4);
-      GO(1, 2, 2, 4);
-    }
-    if (four) GO(1, 4, 8, 2);        // many: 128 a workgroup, which halves the activation traffic
-    GO(1, 2, 8, 2);
+    if (N < 8192) GO3(1, 2, 4, 2, 4, 2, 4);    // 32 weight rows a workgroup, K cut four ways inside it
+    if (M <= 8) GO(1, 1, 4, 2);                // the head: 64 weight rows, or 128 with two passes' worth of rows
+    if (M <= 32) GO(1, 2, 8, 2);
+    GO(1, 4, 8, 2);
   }
-  if constexpr (EPI == EPI_QKV_ROPE) {  // few rows again: one tile a workgroup, K cut eight ways
-    if (four) GO(1, 4, 1, 8);
-    GO(1, 2, 1, 8);
+  if constexpr (EPI == EPI_QKV_ROPE) {
+    const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
+    if (tiles < 256) GO3(1, 1, 8, 1, 8, 1, 8);   // one 16-row tile a workgroup, K cut eight ways
+    GO3(1, 2, 2, 2, 4, 2, 4);                    // two tiles
   }
   if constexpr (EPI == EPI_SWIGLU) {
-    if (four) GO(2, 4, 2, 2);
-    GO(2, 2, 2, 2);
+    const int tiles = (N + 15) / 16;             // N: rows of the gate (and of the up) matrix
+    if (tiles < 768) GO3(2, 1, 8, 2, 2, 2, 2);   // 32 to 64 weight rows a workgroup
+    GO3(2, 4, 2, 4, 2, 4, 2);                    // 128
   }
+#undef GO3
 #undef GO
   return SA_ERR_ARG;
 }
@@ -556,7 +577,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int M, int N, in
 template <typename TC, int EPI>
 static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int K, int up_offset,
                        int parts, const QkvRopeArgs& qa, hipStream_t stream) {
-  // up to 16 rows of activations (more take the kernel above; still more would loop over grid.y).
+  // one or two rows of activations, eight for a small fused q/k/v product (more take the kernel above).
   // Many weight rows: 2 row tiles per wave and few waves; few rows: more waves splitting K.
 #define GO(RT, MT, KS, KU) \
   return launch_skinny<RT, MT, KS, KU, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
@@ -583,7 +604,7 @@ extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || parts < 1) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
-  if (M > 16) {
+  if (!takes_skinny<float, EPI_PLAIN>(M, N, none)) {
     if (c_dtype == SA_BF16 && parts == 1) return pick_mid<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
     if (c_dtype == SA_F32) return pick_mid<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
     return SA_ERR_UNSUPPORTED;
@@ -599,7 +620,7 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
   if (M <= 0 || I <= 0) return 0;
   if (K <= 0 || (K & 7)) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
-  if (M > 16) return pick_mid<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
+  if (!takes_skinny<bf16_t, EPI_SWIGLU>(M, I, none)) return pick_mid<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   return pick_skinny<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
 }
 
@@ -612,6 +633,6 @@ extern "C" int sa_gemm_bf16_qkv_rope(const void* A, const void* W, void* Q, cons
   if (M <= 0) return 0;
   if (K <= 0 || (K & 7) || Hq <= 0 || Hk <= 0 || D <= 0 || (D & 15) || page_size <= 0) return SA_ERR_ARG;
   const QkvRopeArgs qa = {positions, inv_freq, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size};
-  if (M > 16) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
+  if (!takes_skinny<bf16_t, EPI_QKV_ROPE>(M, 0, qa)) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   return pick_skinny<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
 }

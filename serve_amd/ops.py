@@ -277,13 +277,13 @@ def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tor
 
 def split_k_parts(M: int, N: int, K: int) -> int:
     """Into how many slices the inner dimension of a few-row product is cut across workgroups so
-    that a matrix with few rows still fills the chip: 1 means no cut.  Up to 16 rows a workgroup
-    takes 16 weight rows (about 1024 workgroups wanted, slices of at least 256); from 17 rows on it
-    takes 32 (one workgroup per compute unit wanted, slices of at least 512)."""
+    that a matrix with few rows still fills the chip: 1 means no cut.  One or two rows: a workgroup
+    takes 16 weight rows (about 1024 workgroups wanted, slices of at least 256); from three rows on
+    it takes 32 (one workgroup per compute unit wanted, slices of at least 512)."""
     if N >= 8192:
         return 1
     parts = 1
-    if M > 16:
+    if M > 2:
         groups = -(-N // 32)
         while parts < 8 and groups * parts < 256 and K // (parts * 2) >= 512:
             parts *= 2

@@ -459,7 +459,8 @@ def test_prompt_attention_long_prompts_windows_and_split_keys(Hq, Hk, D, ps):
 
 @pytest.mark.parametrize("c_dt", ["bfloat16", "float32"])
 @pytest.mark.parametrize("M,N,K", [(1, 70, 40), (3, 64, 64), (8, 3072, 2048), (16, 509, 96), (17, 130, 104),
-                                   (33, 2048, 8192), (64, 8200, 256), (100, 77, 1024), (8, 128256 // 8, 192)])
+                                   (33, 2048, 8192), (64, 8200, 256), (100, 77, 1024), (8, 128256 // 8, 192),
+                                   (2, 8200, 72), (5, 9001, 64), (24, 8193, 520), (12, 520, 1032)])
 def test_gemm_bf16_skinny(c_dt, M, N, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 4)
@@ -475,7 +476,10 @@ def test_gemm_bf16_skinny(c_dt, M, N, K):
     torch.testing.assert_close(out2.double(), want, **t)
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 192, 64), (8, 8192, 2048), (20, 320, 192), (64, 1000, 96), (50, 8192, 2048)])
+@pytest.mark.parametrize("M,I,K", [(1, 192, 64), (8, 8192, 2048), (20, 320, 192), (64, 1000, 96), (50, 8192, 2048),
+                                   (2, 1000, 72), (3, 1000, 72), (16, 8200, 264), (30, 520, 1032),
+                                   # many rows of weights: 128 of them a workgroup
+                                   (1, 12300, 64), (7, 12300, 264), (24, 14336, 128), (64, 12296, 72)])
 def test_swiglu_bf16(M, I, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 6)
@@ -543,7 +547,10 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
 
 @pytest.mark.parametrize("M,Hq,Hk,D,ps,d", [(1, 4, 2, 32, 8, 64), (8, 32, 8, 64, 16, 2048), (13, 3, 1, 96, 4, 72),
                                              (40, 6, 2, 128, 16, 200), (64, 2, 2, 64, 32, 96), (16, 5, 1, 64, 8, 520), (9, 2, 2, 48, 8, 64),
-                                             (33, 3, 1, 80, 16, 104), (5, 4, 4, 16, 4, 40)])
+                                             (33, 3, 1, 80, 16, 104), (5, 4, 4, 16, 4, 40),
+                                             # 256 tiles of 16 rows and more: two tiles a workgroup
+                                             (1, 24, 8, 128, 16, 136), (8, 32, 8, 128, 16, 520), (20, 24, 4, 128, 8, 72),
+                                             (64, 28, 2, 128, 16, 264), (3, 60, 4, 64, 16, 64)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
     P = 7

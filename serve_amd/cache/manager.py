@@ -131,12 +131,10 @@ class CacheManager:
         """Per group: pages that `ensure(req_id, n_tokens)` would take (0 for an unknown request
         means: as if it were new)."""
         r = self._requests.get(req_id)
-        need_idx = self.pages_for_tokens(n_tokens)
-        out = []
-        for g in range(self.num_groups):
-            have = len(r.tables[g]) if r else 0
-            out.append(max(0, need_idx - have))
-        return out
+        need_idx = -(-n_tokens // self.page_size)
+        if r is None:
+            return [need_idx] * len(self.windows)
+        return [max(0, need_idx - len(t)) for t in r.tables]
 
     # -- changes --------------------------------------------------------------------------------
     def admit(self, req_id) -> Optional[int]:

@@ -80,7 +80,8 @@ class Scheduler:
     token_indices) -> tokens`.
     """
 
-    def __init__(self, runner, sampler, cfg: EngineConfig, eos_token_ids: Optional[Sequence[int]] = None):
+    def __init__(self, runner, sampler, cfg: EngineConfig, eos_token_ids: Optional[Sequence[int]] = None,
+                 record_steps: bool = False):
         self.runner, self.sampler, self.cfg = runner, sampler, cfg
         self.cache = runner.cache
         self.eos = set(eos_token_ids or ())
@@ -90,7 +91,9 @@ class Scheduler:
         self._reserved = [0] * self.cache.num_groups
         self._reservation = {}
         self.steps = 0
-        self.step_log: List[dict] = []       # one record per step, for tests and tracing
+        # one record per step (requests, token counts, who was sampled) when asked for: tracing only
+        self.record_steps = record_steps
+        self.step_log: List[dict] = []
         # decode steps whose tokens are still on the device: the host runs one step ahead
         self._inflight = None
         self.async_decode = (bool(getattr(cfg, "async_decode", True)) and hasattr(runner, "decode_launch")
@@ -170,10 +173,13 @@ class Scheduler:
             plan = StepPlan([], [], [])
             short = None                      # a running request whose portion found no pages
 
+            pages_needed = self.cache.pages_needed
+
             def try_add(r: GenerationRequest, n: int) -> bool:
-                need = self.cache.pages_needed(r.req_id, r.fed + n)
-                if any(need[g] > free[g] for g in range(G)):
-                    return False
+                need = pages_needed(r.req_id, r.fed + n)
+                for g in range(G):
+                    if need[g] > free[g]:
+                        return False
                 for g in range(G):
                     free[g] -= need[g]
                 plan.requests.append(r)
@@ -275,8 +281,7 @@ class Scheduler:
         samplers = [r for r, s in zip(plan.requests, plan.samples) if s]
         tokens = self.sampler.sample(logits, [r.temperature for r in samplers],
                                      [r.req_id for r in samplers], [len(r.generated) for r in samplers])
-        self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in plan.requests],
-                                  counts=list(plan.counts), sampled=[r.req_id for r in samplers]))
+        self._record(plan.requests, plan.counts, samplers)
         self.steps += 1
         for r, n in zip(plan.requests, plan.counts):
             r.fed += n
@@ -324,8 +329,7 @@ class Scheduler:
         handle = self.runner.step_launch([r.req_id for r in reqs], tokens, plan.samples,
                                          [r.temperature for r in samplers], keys)
         previous, self._inflight = self._inflight, (handle, samplers, [len(r.generated) for r in samplers])
-        self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in reqs], counts=list(plan.counts),
-                                  sampled=[r.req_id for r in samplers]))
+        self._record(reqs, plan.counts, samplers)
         self.steps += 1
         for r, n in zip(reqs, plan.counts):
             r.fed += n
@@ -343,8 +347,7 @@ class Scheduler:
         keys = row_keys(self.sampler.seed, [r.req_id for r in reqs], [len(r.generated) for r in reqs])
         handle = self.runner.decode_launch([r.req_id for r in reqs], tokens, [r.temperature for r in reqs], keys)
         previous, self._inflight = self._inflight, (handle, list(reqs), [len(r.generated) for r in reqs])
-        self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in reqs], counts=[1] * len(reqs),
-                                  sampled=[r.req_id for r in reqs]))
+        self._record(reqs, plan.counts, reqs)
         self.steps += 1
         for r in reqs:
             r.fed += 1
@@ -353,6 +356,11 @@ class Scheduler:
                 self._finish(r)               # its pages may go to a later launch, which runs after this one
         if previous is not None:
             self._read_back(previous)
+
+    def _record(self, reqs, counts, samplers) -> None:
+        if self.record_steps:
+            self.step_log.append(dict(step=self.steps, requests=[r.req_id for r in reqs], counts=list(counts),
+                                      sampled=[r.req_id for r in samplers]))
 
     def _read_back(self, flight) -> None:
         handle, reqs, places = flight

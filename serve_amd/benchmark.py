@@ -49,16 +49,18 @@ SHAPES = {
 
 
 def generate_requests(input_length: int, output_length: int, num_sequences: int, vocab_size: int,
-                      fixed_lengths: bool = False, seed: int = 1352):
+                      fixed_lengths: bool = False, seed: int = 1352, min_input_length: int = 1,
+                      fixed_output_length: bool = False):
     """serve/benchmark.py:12-24: lengths uniform in 1..input_length / 1..output_length, ids below
-    10000, seed 1352."""
+    10000, seed 1352.  `min_input_length` raises the lower end of the prompt lengths,
+    `fixed_output_length` gives every request exactly `output_length` new tokens."""
     from .engine.engine import Request
     random.seed(seed)
     torch.manual_seed(seed)
     reqs = []
     for _ in range(num_sequences):
-        n_in = input_length if fixed_lengths else random.randint(1, input_length)
-        n_out = output_length if fixed_lengths else random.randint(1, output_length)
+        n_in = input_length if fixed_lengths else random.randint(min_input_length, input_length)
+        n_out = output_length if fixed_lengths or fixed_output_length else random.randint(1, output_length)
         ids = torch.randint(0, min(10000, vocab_size), (n_in,), dtype=torch.long)
         reqs.append(Request(input_ids=ids, input_length=n_in, max_new_tokens=n_out))
     return reqs
@@ -79,6 +81,8 @@ def main(argv=None) -> int:
     ap.add_argument("--num-sequences", type=int, default=2000)
     ap.add_argument("--temperature", type=float, default=0.6)
     ap.add_argument("--fixed-lengths", action="store_true", help="every request has exactly the given lengths")
+    ap.add_argument("--min-input-length", type=int, default=1, help="prompt lengths are uniform from here to --input-length")
+    ap.add_argument("--fixed-output-length", action="store_true", help="every request generates exactly --output-length tokens")
     ap.add_argument("--seed", type=int, default=0, help="seed of the random weights and of the sampler")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--memory-fraction", type=float, default=0.6, help="share of free memory for the cache "
@@ -102,7 +106,8 @@ def main(argv=None) -> int:
         engine = Engine.from_config(SHAPES[args.shape], args.seed, cfg)
     print(f"Model finished loading; cache of {engine.runner.num_pages} pages of {args.page_size} tokens")
     requests = generate_requests(args.input_length, args.output_length, args.num_sequences,
-                                 engine.model.spec.vocab_size, args.fixed_lengths)
+                                 engine.model.spec.vocab_size, args.fixed_lengths,
+                                 min_input_length=args.min_input_length, fixed_output_length=args.fixed_output_length)
 
     def fn():
         return engine.generate(requests, args.temperature)

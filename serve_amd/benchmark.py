@@ -88,7 +88,8 @@ def main(argv=None) -> int:
     ap.add_argument("--memory-fraction", type=float, default=0.6, help="share of free memory for the cache "
                     "(serve/model.py:172)")
     ap.add_argument("--max-context", type=int, default=2048, help="serve/model.py:32")
-    ap.add_argument("--max-requests", type=int, default=256)
+    ap.add_argument("--max-requests", type=int, default=2048, help="requests live at a time at most; the reference "
+                    "admits by cache capacity alone (serve/run.py:267-280)")
     ap.add_argument("--max-tokens-per-step", type=int, default=2048, help="serve/run.py:265")
     ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")

@@ -1000,7 +1000,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   }
   if (small) {
     // single decoded tokens (at most 16 rows per KV head): one wave per (segment, KV head, split)
-    dim3 grid(1, Hk, B * num_splits), block(256);
+    dim3 grid(1, Hk, B * num_splits), block(64);   // one wave: tile 0 is the only tile of such a segment
     const int pm = page_shift >= 5 ? 2 : (page_shift >= 3 ? 1 : 0);
 #define GO(PM)                                                                                         \
   hipLaunchKernelGGL((paged_attention_mfma_kernel<PM>), grid, block, 0, stream,                        \

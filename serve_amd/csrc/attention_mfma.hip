@@ -75,7 +75,7 @@ struct Unmasked { static constexpr bool value = false; };
 //      pages and each lane picks its own;
 //   2  a power of two of at least 32: a block lies in one page, and every address is a scalar base
 //      plus a constant of the lane.
-template <int PM>
+template <int PM, bool LOCAL = false>
 __device__ __forceinline__ void attention_tile(
     const int tile, const int seg, const int hk, const int sp, const int q_begin, const int q_len,
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -389,7 +389,8 @@ __device__ __forceinline__ void attention_tile(
         *reinterpret_cast<uint2*>(op + dt * 16 + 4 * g) = w;
       }
     } else {
-      const size_t slot = ((size_t)tok[n] * Hq + head[n]) * num_splits + sp;
+      // LOCAL: the parts stay in the workgroup (part_o, part_ml lie in LDS), indexed [split][row of the tile]
+      const size_t slot = LOCAL ? (size_t)sp * 16 + c : ((size_t)tok[n] * Hq + head[n]) * num_splits + sp;
       float* po = part_o + slot * HD;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
@@ -418,6 +419,71 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int q_len = cu_q[seg + 1] - q_begin;
   attention_tile<PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table, max_pages,
                      ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits, part_o, part_ml);
+}
+
+// The same for short contexts: the WS waves of a workgroup take the WS parts of the key range of one
+// (segment, KV head) and merge their (m, l, O) through LDS, in the order of the parts, so that no
+// merge kernel follows: out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), an empty part weighs 0.
+// Short contexts only: the keys and values of a (segment, KV head) then pass through one compute unit.
+constexpr int WG_SPLITS = 4;
+
+template <int PM>
+__global__ __launch_bounds__(64 * WG_SPLITS) void paged_attention_mfma_wg_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
+    int window) {
+  __shared__ float part_o[WG_SPLITS * 16 * HD];
+  __shared__ float part_ml[WG_SPLITS * 16 * 2];
+  const int wave = threadIdx.x >> 6;
+  const int hk = blockIdx.y;
+  const int seg = blockIdx.z;
+  const int q_begin = cu_q[seg];
+  const int q_len = cu_q[seg + 1] - q_begin;
+  attention_tile<PM, true>(0, seg, hk, wave, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
+                           max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, WG_SPLITS,
+                           part_o, part_ml);
+  __syncthreads();
+  if (wave != 0) return;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int G = Hq / Hk;
+  if (c >= q_len * G) return;
+  float ms[WG_SPLITS], M = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < WG_SPLITS; ++s) {
+    ms[s] = part_ml[(s * 16 + c) * 2];
+    M = fmaxf(M, ms[s]);
+  }
+  float L = 0.f;
+  floatx4_t o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < WG_SPLITS; ++s) {
+    const float w = ms[s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms[s] - M);
+    L += part_ml[(s * 16 + c) * 2 + 1] * w;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const float4 p = *reinterpret_cast<const float4*>(part_o + (s * 16 + c) * HD + dt * 16 + 4 * g);
+      o[dt][0] += p.x * w;
+      o[dt][1] += p.y * w;
+      o[dt][2] += p.z * w;
+      o[dt][3] += p.w * w;
+    }
+  }
+  const float inv = 1.f / L;
+  const int j = c / G;
+  bf16_t* op = out + ((size_t)(q_begin + j) * Hq + hk * G + (c - j * G)) * HD;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    uint2 w;
+    w.x = pack2bf(o[dt][0] * inv, o[dt][1] * inv);
+    w.y = pack2bf(o[dt][2] * inv, o[dt][3] * inv);
+    *reinterpret_cast<uint2*>(op + dt * 16 + 4 * g) = w;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -978,12 +1044,14 @@ extern "C" int sa_attention_mfma_head_dim() { return HD; }
 constexpr int COMPUTE_UNITS = 256;
 
 // A step whose segments have at most 16 rows each (single decoded tokens) takes the one-wave kernel,
-// any other the prompt kernel.
+// any other the prompt kernel.  `in_workgroup` (such steps only, num_splits 1): the key range of every
+// (segment, KV head) is cut four ways over the waves of one workgroup, which merges the parts itself.
 extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, const void* k_pages,
                                        const void* v_pages, const int* block_table, int max_pages,
                                        const int* cu_q, const int* ctx_len, int B, int T, int max_q_len,
                                        int Hq, int Hk, int D, int page_size, float scale, int window,
-                                       int num_splits, float* part_o, float* part_ml, hipStream_t stream) {
+                                       int num_splits, float* part_o, float* part_ml, int in_workgroup,
+                                       hipStream_t stream) {
   if (T <= 0 || B <= 0) return 0;
   if (D != HD || Hq <= 0 || Hk <= 0 || Hq % Hk || page_size <= 0 || (page_size & 3) || max_pages <= 0 ||
       max_q_len <= 0 || num_splits < 1 || num_splits > 64 || (q_stride & 7))
@@ -997,6 +1065,23 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
+  }
+  if (in_workgroup && (!small || num_splits != 1 || B > 65535)) return SA_ERR_ARG;
+  if (small && in_workgroup) {
+    // the key range cut four ways inside a workgroup and merged there: for short contexts
+    dim3 grid(1, Hk, B), block(64 * WG_SPLITS);
+    const int pm = page_shift >= 5 ? 2 : (page_shift >= 3 ? 1 : 0);
+#define GO(PM)                                                                                         \
+  hipLaunchKernelGGL((paged_attention_mfma_wg_kernel<PM>), grid, block, 0, stream,                     \
+                     (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages,                 \
+                     (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
+                     page_shift, scale_log2e, window)
+    if (pm == 2) GO(2);
+    else if (pm == 1) GO(1);
+    else GO(0);
+#undef GO
+    SA_LAUNCH_CHECK();
+    return 0;
   }
   if (small) {
     // single decoded tokens (at most 16 rows per KV head): one wave per (segment, KV head, split)

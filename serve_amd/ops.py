@@ -394,13 +394,30 @@ def attention_splits(max_q_len: int, num_segments: int, num_kv_heads: int, max_c
     return max(1, min(by_length, by_waves, 64))
 
 
+IN_WORKGROUP_MAX_CTX = 512
+IN_WORKGROUP_MAX_SEGMENTS = 32
+
+
+def attention_in_workgroup(max_q_len: int, num_segments: int, max_ctx_len: int, group_size: int = 1) -> bool:
+    """Whether single decoded tokens have their keys cut inside a workgroup (four waves that merge
+    through LDS, no merge kernel) instead of across workgroups: for few requests with short
+    contexts, where the launch is a chain of latencies and the merge kernel one more link (batch 1
+    to 32 at 384 keys: 5.5 to 7.8 us against 5.9 to 8.5 us; at 64 requests or 1,024 keys the cut
+    across workgroups, or none, is faster).  Both bounds are powers of two, so that a step run
+    eagerly and the same step replayed from a graph (batch and context rounded up to powers of
+    two) decide alike."""
+    return (max_q_len * group_size <= 16 and num_segments <= IN_WORKGROUP_MAX_SEGMENTS
+            and 64 < max_ctx_len <= IN_WORKGROUP_MAX_CTX)
+
+
 def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                          v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                          ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int, scale: float,
                          window: Optional[int], num_splits: int = 1, seg_begin: int = 0,
-                         seg_count: Optional[int] = None) -> torch.Tensor:
+                         seg_count: Optional[int] = None, in_workgroup: bool = False) -> torch.Tensor:
     """bf16 attention on the matrix cores (head sizes 16..128 in steps of 16, page sizes that are
-    multiples of 4).  `seg_begin`, `seg_count`: run only these segments of the step (their
+    multiples of 4).  `in_workgroup` (segments of at most 16 rows per KV head, num_splits 1): the
+    key range is cut four ways over the waves of a workgroup, which merges the parts itself.  `seg_begin`, `seg_count`: run only these segments of the step (their
     tokens' rows of `out` are written, the others left alone); `num_tokens` then is the number of
     tokens up to the end of the last of them."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
@@ -428,6 +445,8 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
         cu_q = cu_q[seg_begin: seg_begin + B + 1]
         ctx_len = ctx_len[seg_begin: seg_begin + B]
     _check(1 <= max_q_len <= max(T, 1) and num_splits >= 1, "max_q_len / num_splits out of range")
+    _check(not in_workgroup or (num_splits == 1 and max_q_len * (num_heads // Hk) <= 16),
+           "the cut inside a workgroup is for segments of at most 16 rows per KV head and takes no other cut")
     part_o = part_ml = None
     if num_splits > 1:
         # the parts are indexed by token, and the merge runs over tokens 0 .. T-1
@@ -439,7 +458,8 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(T), c_int(max_q_len),
         c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0),
-        c_int(num_splits), _ptr(part_o), _ptr(part_ml), _stream()), "paged_attention_mfma")
+        c_int(num_splits), _ptr(part_o), _ptr(part_ml), c_int(1 if in_workgroup else 0), _stream()),
+        "paged_attention_mfma")
     return out
 
 
@@ -483,9 +503,12 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
         # (first segment, segments, tokens up to their end, longest portion, longest context)
         for s0, n, t_end, max_q, max_ctx in _attention_launches(ctx):
             # (the parts of a split key range are indexed by token, from the step's first)
-            splits = attention_splits(max_q, n, Hk, max_ctx, num_heads // Hk) if max_q == 1 or s0 == 0 else 1
+            inside = max_q == 1 and attention_in_workgroup(max_q, n, max_ctx, num_heads // Hk)
+            splits = 1
+            if not inside and (max_q == 1 or s0 == 0):
+                splits = attention_splits(max_q, n, Hk, max_ctx, num_heads // Hk)
             paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
-                                 t_end, max_q, num_heads, scale, window, splits, s0, n)
+                                 t_end, max_q, num_heads, scale, window, splits, s0, n, in_workgroup=inside)
         return out
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                   ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

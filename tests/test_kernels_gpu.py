@@ -178,7 +178,7 @@ def test_rope_depends_on_distance_only():
 
 # ---------------------------------------------------------------------------------------------
 def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False, kernel="simple", splits=1,
-                   poison=False):
+                   poison=False, in_workgroup=False):
     """segs: list of (ctx_before, q_len).  Builds a paged cache with shuffled pages, runs the
     kernel, and compares with dense softmax attention per segment."""
     from serve_amd import ops
@@ -238,7 +238,7 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
         assert len(ctx._attention_launches) == splits          # here: the number of launches expected
     else:
         ops.paged_attention_mfma(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
-                                 max(ql for _, ql in segs), Hq, scale, window, splits)
+                                 max(ql for _, ql in segs), Hq, scale, window, splits, in_workgroup=in_workgroup)
     G = Hq // Hk
     for i, (c, ql) in enumerate(segs):
         qi = q[cu[i]: cu[i + 1]].double().view(ql, Hq, D)
@@ -362,6 +362,13 @@ def test_paged_attention_mfma_mixed(Hq, Hk, D, ps):
 def test_paged_attention_mfma_decode_with_splits(Hq, Hk, D, ps, splits):
     segs = [(12, 1), (0, 1), (130, 1), (517, 1), (31, 1), (32, 1), (63, 1), (64, 1)]
     attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=300 + D, kernel="mfma", splits=splits)
+    # the same contexts with the keys cut inside a workgroup (four waves that merge through LDS),
+    # also with segments of a few tokens that still fit one 16-row tile, a window, and NaN beyond the context
+    attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=320 + D, kernel="mfma", in_workgroup=True)
+    few = [(40, 16 // (Hq // Hk)), (0, 2), (300, 1), (95, 1), (96, 1), (127, 1), (128, 1)]
+    attention_case("bfloat16", Hq, Hk, D, ps, few, seed=321 + D, kernel="mfma", in_workgroup=True)
+    attention_case("bfloat16", Hq, Hk, D, ps, segs, seed=322 + D, kernel="mfma", in_workgroup=True, window=40,
+                   poison=True)
 
 
 @pytest.mark.parametrize("Hq,Hk,D,ps", [(8, 2, 64, 16), (6, 2, 128, 16), (3, 1, 32, 8), (4, 4, 48, 12)])

@@ -11,9 +11,11 @@
 // attn_decode.py:341-348, has none and is switched off).
 //
 // The rows of a segment are its (token, query head of the group) pairs, row = token * G +
-// head_in_group, so the G heads that share a KV head share every K and V load.  Two kernels: one
-// wave per (segment, KV head, split of the key range) for single decoded tokens, workgroups that
-// share K and V through LDS for prompt portions.
+// head_in_group, so the G heads that share a KV head share every K and V load.  Single decoded
+// tokens take one wave per (segment, KV head, split of the key range), as workgroups of one wave
+// whose parts a merge kernel joins, or, for few requests with short contexts, as workgroups of four
+// waves that join their parts through LDS; prompt portions take workgroups that share K and V
+// through LDS.
 //
 // MFMA use (v_mfma_f32_16x16x32_bf16: D[i][j] += sum_k A[i][k] B[k][j]; lane l holds A row l%16,
 // B column l%16, k-slots 8*(l/16)..+7, and D[4*(l/16)+r][l%16]):

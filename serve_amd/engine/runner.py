@@ -260,7 +260,9 @@ class ModelRunner:
         place; `temperatures` and `keys` belong to those requests, in order, and so do the tokens
         of the handle."""
         with torch.cuda.device(self.rt.device):
-            segments = [Segment(r, [0 if t is None else t for t in toks], [len(toks) - 1] if smp else [])
+            if any(toks[0] is None and len(toks) != 1 for toks in tokens):
+                raise ValueError("only a single token can be left to the device")
+            segments = [Segment(r, toks if toks[0] is not None else [0], [len(toks) - 1] if smp else [])
                         for r, toks, smp in zip(req_ids, tokens, samples)]
             lay, host, facts = plan_step(segments, self.cache, self.vocab_size)
             T, R = lay.T, lay.R
@@ -275,8 +277,6 @@ class ModelRunner:
             cu = host[lay.cu_q: lay.cu_q + len(segments)]
             for i, (r, toks) in enumerate(zip(req_ids, tokens)):
                 if toks[0] is None:
-                    if len(toks) != 1:
-                        raise ValueError("only a single token can be left to the device")
                     src[cu[i]] = self._row_of[r]
             buf[off_temps: off_temps + R].view(np.float32)[:] = np.asarray(temperatures, dtype=np.float32)
             buf[off_keys: off_keys + 2 * R].view(np.int64)[:] = np.asarray(keys, dtype=np.int64)

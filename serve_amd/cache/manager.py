@@ -62,6 +62,7 @@ class _Request:
     slot: int
     tokens: int = 0                                                  # tokens the tables cover
     tables: List[List[int]] = field(default_factory=list)            # per group: page per index
+    covered: int = 0                                                 # pages every group's table has
 
 
 class CacheManager:
@@ -84,6 +85,7 @@ class CacheManager:
         self.max_requests = max_requests
         self.max_pages_per_request = max_pages_per_request
         self.pools = [PagePool(n) for n in num_pages]
+        self._none_needed = [0] * len(windows)    # (shared, read only)
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
         self._requests: Dict[object, _Request] = {}
         # the block tables once more as one int32 matrix per group, row = state slot, so that a
@@ -134,6 +136,8 @@ class CacheManager:
         need_idx = -(-n_tokens // self.page_size)
         if r is None:
             return [need_idx] * len(self.windows)
+        if need_idx <= r.covered:
+            return self._none_needed
         return [max(0, need_idx - len(t)) for t in r.tables]
 
     # -- changes --------------------------------------------------------------------------------
@@ -151,7 +155,11 @@ class CacheManager:
         """Grow the request's block tables to cover `n_tokens` tokens.  All or nothing: on False
         nothing has changed."""
         r = self._requests[req_id]
-        need_idx = self.pages_for_tokens(n_tokens)
+        need_idx = -(-n_tokens // self.page_size)
+        if need_idx <= r.covered:                 # the usual case of a decoded token: its page is there
+            if n_tokens > r.tokens:
+                r.tokens = n_tokens
+            return True
         if need_idx > self.max_pages_per_request:
             raise CacheError(f"request {req_id!r} needs {need_idx} pages, above the limit of "
                              f"{self.max_pages_per_request} per request (max_context)")
@@ -165,6 +173,7 @@ class CacheManager:
                 r.tables[g].extend(new)
                 self.table_rows[g][r.slot, have: have + w] = new
         r.tokens = max(r.tokens, n_tokens)
+        r.covered = min((len(t) for t in r.tables), default=self.max_pages_per_request)
         return True
 
     def trim(self, req_id, n_tokens_done: int) -> int:
@@ -213,6 +222,9 @@ class CacheManager:
             for r in self._requests.values():
                 if self.table_rows[g][r.slot, : len(r.tables[g])].tolist() != r.tables[g]:
                     raise CacheError(f"group {g}: the table matrix and the table of a request differ")
+        for r in self._requests.values():
+            if r.tables and r.covered != min(len(t) for t in r.tables):
+                raise CacheError("the count of pages that every group covers is stale")
         slots = [r.slot for r in self._requests.values()]
         if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots):
             raise CacheError("a state slot is held twice")

@@ -407,7 +407,7 @@ def attention_in_workgroup(max_q_len: int, num_segments: int, max_ctx_len: int, 
     pages by itself and lost 2 % in the decode step).  Batch and context are rounded up to powers
     of two first, so that a step run eagerly and the same step replayed from a graph (which rounds
     both) decide alike."""
-    if max_q_len * group_size > 16 or max_ctx_len <= 64:
+    if max_q_len * group_size > 16:
         return False
     segs = 1
     while segs < num_segments:

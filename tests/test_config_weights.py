@@ -243,3 +243,23 @@ def test_named_shapes_are_the_configurations_the_measurements_are_specified_on()
     assert SHAPES["llama-3b"].num_hidden_layers == 28 and SHAPES["llama-8b"].intermediate_size == 14336
     for cfg in SHAPES.values():
         cfg.validate()
+
+
+def test_attention_launch_policy_is_the_same_for_a_step_and_its_graph_replay():
+    """A decode step replayed from a graph sees its batch padded to the next captured size and its
+    longest context rounded up to a power of two; the choice of key splits and of the cut inside a
+    workgroup must not change with that, or a replay would differ from the eager step."""
+    import random
+    from serve_amd import ops
+    from serve_amd.engine.runner import GRAPH_BATCHES
+    rng = random.Random(5)
+    for _ in range(2000):
+        B = rng.randrange(1, GRAPH_BATCHES[-1] + 1)
+        ctx = rng.randrange(1, 140000)
+        Hk, G = rng.choice([1, 2, 4, 8]), rng.choice([1, 3, 4, 8])
+        b_pad = next(b for b in GRAPH_BATCHES if b >= B)
+        bucket = 256
+        while bucket < ctx:
+            bucket *= 2
+        assert ops.attention_splits(1, B, Hk, ctx, G) == ops.attention_splits(1, b_pad, Hk, bucket, G)
+        assert ops.attention_in_workgroup(1, B, ctx, G) == ops.attention_in_workgroup(1, b_pad, bucket, G)

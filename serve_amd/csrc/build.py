@@ -31,6 +31,8 @@ FLAGS = [
     "-Wno-unused-command-line-argument",
 ]
 HEADERS = ["common.h"]
+# headers that only one source includes (its C interface)
+OWN_HEADERS: Dict[str, List[str]] = {"sampling.hip": ["sampling.h"]}
 
 # library name -> source file; variants (same source, other defines) are named on request
 SOURCES: Dict[str, str] = {
@@ -93,7 +95,7 @@ def _search_dirs() -> List[str]:
 
 def _key(source: str, defines: Tuple[Tuple[str, str], ...]) -> str:
     h = hashlib.sha256()
-    for name in [source] + HEADERS:
+    for name in [source] + HEADERS + OWN_HEADERS.get(source, []):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(FLAGS).encode())

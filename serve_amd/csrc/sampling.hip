@@ -7,6 +7,9 @@
 // and the vocabulary index, so a request's draws do not depend on what else is in the batch.
 // Ties go to the lowest index.
 #include "common.h"
+#include "sampling.h"
+
+#include <mutex>
 
 __device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
   z += 0x9E3779B97F4A7C15ull;
@@ -106,4 +109,60 @@ extern "C" int sa_sample(const float* logits, const float* temperature, const un
   hipLaunchKernelGGL(sample_final_kernel, dim3(R), dim3(64), 0, stream, part_v, part_i, out, nchunks);
   SA_LAUNCH_CHECK();
   return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same two kernels with their partial results in an array of the library's own, for callers
+// that cannot allocate (see sampling.h).  `scratch` is a device symbol: in host code its name is
+// only a stand-in, the array's address on a device comes from hipGetSymbolAddress, once per
+// device (every GPU holds its own copy of the array at its own address).
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[SA_SAMPLE_NOALLOC_ENTRIES * 8];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// the address of `scratch` on the current device; 0 and *err set if the lookup fails
+void* scratch_on_current_device(int* err) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    *err = (int)e;
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    *err = SA_ERR_ARG;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      *err = e != hipSuccess ? (int)e : SA_ERR_ARG;
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int sa_sample_noalloc_max_entries(void) { return SA_SAMPLE_NOALLOC_ENTRIES; }
+
+extern "C" int sa_sample_noalloc(const float* logits, const float* temperature, const unsigned long long* keys,
+                                 int* out, int R, int V, hipStream_t stream) {
+  if (R <= 0) return 0;
+  if (V <= 0 || R > 65535 || !logits || !out) return SA_ERR_ARG;
+  const long long entries = (long long)R * sa_sample_chunks(V);
+  if (entries > SA_SAMPLE_NOALLOC_ENTRIES) return SA_ERR_ARG;
+  int err = 0;
+  void* base = scratch_on_current_device(&err);
+  if (!base) return err;
+  // first half: the chunks' best scores, second half: their indices
+  float* part_v = reinterpret_cast<float*>(base);
+  int* part_i = reinterpret_cast<int*>(static_cast<unsigned char*>(base) + (size_t)SA_SAMPLE_NOALLOC_ENTRIES * 4);
+  return sa_sample(logits, temperature, keys, out, part_v, part_i, R, V, stream);
 }

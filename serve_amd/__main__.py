@@ -29,6 +29,9 @@ def _generate(argv) -> int:
                     "instead of --prompt-ids")
     ap.add_argument("--max-new-tokens", type=int, default=32)
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy (serve/run.py:56-57)")
+    ap.add_argument("--stop-at-eos", action="store_true", help="a request ends with the first end-of-sequence token "
+                    "(config.json's eos_token_id) it generates; default: at --max-new-tokens only (serve/run.py:222)")
+    ap.add_argument("--stop-token-ids", type=int, nargs="+", metavar="ID", help="token ids that end a request")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=None)
@@ -69,11 +72,20 @@ def _generate(argv) -> int:
             line = line.strip()
             if line:
                 prompts.append(json.loads(line) if line.startswith("[") else [int(t) for t in line.split()])
+    stop = None
+    if args.stop_at_eos or args.stop_token_ids:
+        stop = list(args.stop_token_ids or [])
+        if args.stop_at_eos:
+            stop += engine.stop_ids("eos")
     out = engine.generate([Request(torch.tensor(p, dtype=torch.long), len(p), args.max_new_tokens) for p in prompts],
-                          temperature=args.temperature)
-    for r in out:
+                          temperature=args.temperature, stop_token_ids=stop)
+    failed = 0
+    for i, r in enumerate(out):
         print(json.dumps(r.generated_tokens.tolist()), flush=True)
-    return 0
+        if r.error:
+            failed += 1
+            print(f"request {i} did not run: {r.error}", file=sys.stderr, flush=True)
+    return 1 if failed else 0
 
 
 def _random_model(argv) -> int:
@@ -83,7 +95,11 @@ def _random_model(argv) -> int:
     g.add_argument("--shape", help="a named shape (tiny, tiny-a, tiny-b, llama-1b, llama-3b, llama-8b)")
     g.add_argument("--config", help="a config.json to take the sizes from")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--weight-dtype", choices=["bfloat16", "float32"], default="bfloat16",
+                    help="the dtype the tensors are stored in")
     args = ap.parse_args(argv)
+    import torch
+
     from .weights.loader import write_random_model
     if args.shape:
         from .benchmark import SHAPES
@@ -95,7 +111,7 @@ def _random_model(argv) -> int:
         with open(args.config) as f:
             raw = json.load(f)
         config = get_architecture(raw["architectures"][0]).config_from_dict(raw)
-    write_random_model(args.out, config, args.seed)
+    write_random_model(args.out, config, args.seed, getattr(torch, args.weight_dtype))
     print(args.out)
     return 0
 

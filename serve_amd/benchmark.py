@@ -125,6 +125,11 @@ def main(argv=None) -> int:
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - st
         total = sum(len(r.generated_tokens) for r in responses)
+        failed = [(i, r.error) for i, r in enumerate(responses) if r.error]
+        if failed:
+            print(f"{len(failed)} requests did not run; the first: request {failed[0][0]}: {failed[0][1]}",
+                  file=sys.stderr)
+            return 1
         print(f"Time taken: {elapsed:.4f} seconds")
         print(f"Throughput: {total / elapsed:.2f} tokens/second")
     if args.profile or args.profile_only:

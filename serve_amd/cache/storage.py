@@ -1,9 +1,11 @@
 """Device memory of the cache: page tensors per cache layer and state rows per request.
 
-Layout of one layer's pages (the reference keeps `[NB, bs, D]` per KV head,
-serve/model.py:176-182): keys `[P, Hk, page_size, D]` so that one head's keys of a page are
-contiguous rows, values `[P, Hk, D, page_size]` (transposed inside the page) so that the
-matrix-core product P.V reads runs of consecutive keys at a fixed dim.
+What a layer keeps per token is the mixer's to say (`TokenCacheRequest`: named tensors with a
+per-token shape and the axis along which a page's tokens lie).  The framework's attention
+keeps keys `[P, Hk, page_size, D]`, so that one head's keys of a page are contiguous rows,
+and values `[P, Hk, D, page_size]` (transposed inside the page), so that the matrix-core
+product P.V reads runs of consecutive keys at a fixed dim (the reference keeps `[NB, bs, D]`
+per KV head for both, serve/model.py:176-182).
 """
 from __future__ import annotations
 
@@ -11,10 +13,10 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from ..parts.base import KVCacheRequest, LayerCache, Runtime, StateRequest
+from ..parts.base import LayerCache, Runtime, StateRequest, TokenCacheRequest
 
 
-def group_windows(requests: Sequence[Optional[KVCacheRequest]]) -> List[Optional[int]]:
+def group_windows(requests: Sequence[Optional[TokenCacheRequest]]) -> List[Optional[int]]:
     """The distinct retention rules of the model's cache layers, full retention first."""
     seen: List[Optional[int]] = []
     for r in requests:
@@ -24,18 +26,24 @@ def group_windows(requests: Sequence[Optional[KVCacheRequest]]) -> List[Optional
     return seen
 
 
-def bytes_per_page(requests: Sequence[Optional[KVCacheRequest]], windows: Sequence[Optional[int]],
-                   page_size: int, itemsize: int) -> List[int]:
-    """Per group: bytes that one page id costs over all layers of the group."""
+def _itemsize(dtype: torch.dtype) -> int:
+    return torch.empty((), dtype=dtype).element_size()
+
+
+def bytes_per_page(requests: Sequence[Optional[TokenCacheRequest]], windows: Sequence[Optional[int]],
+                   page_size: int, dtype: torch.dtype) -> List[int]:
+    """Per group: bytes that one page id costs over all layers of the group (`dtype` is the
+    activation dtype, which a cache tensor without a dtype of its own takes)."""
     out = [0] * len(windows)
     for r in requests:
         if r is not None:
-            out[windows.index(r.window)] += 2 * r.num_kv_heads * r.head_dim * page_size * itemsize
+            for t in r.tensors:
+                out[windows.index(r.window)] += t.elements_per_token() * page_size * _itemsize(t.dtype or dtype)
     return out
 
 
 class CacheStorage:
-    def __init__(self, rt: Runtime, cache_requests: Sequence[Optional[KVCacheRequest]],
+    def __init__(self, rt: Runtime, cache_requests: Sequence[Optional[TokenCacheRequest]],
                  state_requests: Sequence[Optional[StateRequest]], windows: Sequence[Optional[int]],
                  num_pages: Sequence[int], page_size: int, max_requests: int):
         self.layers: List[LayerCache] = []
@@ -44,12 +52,14 @@ class CacheStorage:
             if cr is not None:
                 g = list(windows).index(cr.window)
                 lc.group = g
-                # zero-filled: an unwritten slot must not hold NaN bit patterns, which 0 * NaN
-                # would carry into a masked position's product
-                lc.k_pages = torch.zeros((num_pages[g], cr.num_kv_heads, page_size, cr.head_dim),
-                                         dtype=rt.dtype, device=rt.device)
-                lc.v_pages = torch.zeros((num_pages[g], cr.num_kv_heads, cr.head_dim, page_size),
-                                         dtype=rt.dtype, device=rt.device)
+                names = [t.name for t in cr.tensors]
+                if len(set(names)) != len(names):
+                    raise ValueError(f"a cache request names a tensor twice: {names}")
+                for t in cr.tensors:
+                    # zero-filled: an unwritten slot must not hold NaN bit patterns, which 0 * NaN
+                    # would carry into a masked position's product
+                    lc.pages[t.name] = torch.zeros((num_pages[g],) + t.page_shape(page_size),
+                                                   dtype=t.dtype or rt.dtype, device=rt.device)
             if sr is not None:
                 lc.state = torch.zeros((max_requests,) + tuple(sr.shape), dtype=sr.dtype, device=rt.device)
             self.layers.append(lc)

@@ -22,16 +22,16 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer = an arrangement of a mixer and a feed-forward with their norms.
+    """One layer = an arrangement and the parts it is made of, by name.
 
-    `weights` maps the local tensor names of the layer's parts (`mixer.q_proj.weight`,
-    `ffn.gate_proj.weight`, `mixer_norm.weight`, ...) to tensor names in the checkpoint.
+    Which names a layer has, and which role each plays (mixer, feed_forward, norm), is the
+    arrangement's business: `prenorm_residual` takes `mixer`, `ffn`, `mixer_norm` and `ffn_norm`;
+    an arrangement with four norms, or none, names its own.  `weights` maps the local tensor
+    names of the layer's parts (`mixer.q_proj.weight`, `ffn.gate_proj.weight`,
+    `mixer_norm.weight`, ...) to tensor names in the checkpoint.
     """
 
-    mixer: PartSpec
-    ffn: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    parts: Dict[str, PartSpec]
     weights: Dict[str, str]
     arrangement: str = "prenorm_residual"
 

@@ -107,7 +107,8 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
 
     Returns (layout, host int32 array, host facts).  Raises `OutOfPages` before anything is
     allocated if the pools cannot cover the whole step.  `pad_segments_to` appends inert
-    one-token segments (no cache write) so that a step has a fixed shape for graph replay.
+    one-token segments (cache slot -1: nothing stored; state slot -1: no request's state) so that
+    a step has a fixed shape for graph replay.
     """
     if not segments:
         raise ValueError("a step needs at least one segment")
@@ -171,6 +172,7 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         host[lay.cu_q: lay.cu_q + B + 1] = np.arange(B + 1)
         host[lay.ctx_len: lay.ctx_len + B] = 1
         host[lay.ctx_len: lay.ctx_len + n] = before_np + 1
+        host[lay.state_slots: lay.state_slots + B] = -1          # padding rows belong to no request
         host[lay.state_slots: lay.state_slots + n] = slots_np
         host[lay.logit_rows: lay.logit_rows + R] = [i for i, s in enumerate(segments) if len(s.want)]
         for g in range(G):
@@ -225,6 +227,7 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         host[lay.seg_of_token + cu] = i
         host[lay.cu_q + i] = cu
         host[lay.ctx_len + i] = 1
+        host[lay.state_slots + i] = -1
         for g in range(G):
             host[lay.slots[g] + cu] = -1
         cu += 1

@@ -33,6 +33,9 @@ class Request:
     max_new_tokens: int
     generated_tokens: torch.Tensor = field(default_factory=lambda: torch.tensor([], dtype=torch.long))
     logits: Optional[torch.Tensor] = None
+    # why the request ended without (all of) its tokens: it exceeds max_context, does not fit into
+    # the cache, has an empty prompt; None when it ran to its end
+    error: Optional[str] = None
 
 
 def _dtype_name(dtype) -> str:
@@ -59,7 +62,7 @@ class Engine:
     def _build(arch, config, reader, cfg: EngineConfig) -> "Engine":
         cfg.validate()
         device = require_gpu(cfg.device)
-        rt = Runtime(device, _TORCH_DTYPE[cfg.dtype])
+        rt = Runtime(device, _TORCH_DTYPE[cfg.dtype], max_context=cfg.max_context)
         model = Model(arch.build_spec(config))
         with torch.cuda.device(device):
             load_weights(model, reader(model) if callable(reader) else reader, rt)
@@ -83,13 +86,37 @@ class Engine:
     def step(self, segments) -> torch.Tensor:
         return self.runner.step(segments)
 
+    def stop_ids(self, stop_token_ids) -> Optional[List[int]]:
+        """None; "eos": the end-of-sequence ids of the model's configuration; or a list of ids."""
+        if stop_token_ids is None:
+            return None
+        if isinstance(stop_token_ids, str):
+            if stop_token_ids != "eos":
+                raise ValueError(f"stop_token_ids must be None, 'eos' or a list of token ids, not {stop_token_ids!r}")
+            ids = self.model.spec.eos_token_ids
+            if not ids:
+                raise ValueError("stop_token_ids='eos': the model's configuration names no eos_token_id")
+            return list(ids)
+        ids = [int(t) for t in stop_token_ids]
+        for t in ids:
+            if not 0 <= t < self.model.spec.vocab_size:
+                raise ValueError(f"stop token {t} is outside the vocabulary [0, {self.model.spec.vocab_size})")
+        return ids
+
     def generate(self, requests: Sequence[Request], temperature: Union[float, Sequence[float]] = 0.0,
-                 return_logits: Union[bool, str] = False) -> List[Request]:
-        """Generate `max_new_tokens` tokens for every request; results in the order given
+                 return_logits: Union[bool, str] = False, stop_token_ids=None,
+                 raise_on_error: bool = False) -> List[Request]:
+        """Generate up to `max_new_tokens` tokens for every request; results in the order given
         (serve/run.py:304).  `temperature` 0 is greedy (serve/run.py:56-57); one value for all
         requests as in the reference, or one per request.  `return_logits`: False / "none"; True /
         "last": the fp32 logits [V] that the last token was drawn from, as the reference returns
-        them (serve/run.py:229-230); "all": those of every generated token, [generated, V]."""
+        them (serve/run.py:229-230); "all": those of every generated token, [generated, V].
+        `stop_token_ids`: None (the reference's behaviour: a request ends at `max_new_tokens`
+        only, serve/run.py:222), "eos" (the configuration's end-of-sequence ids) or a list of
+        ids; a request ends with the first of them it generates, which stays in its tokens.
+        A request that cannot run (longer than max_context, larger than the cache, empty) comes
+        back with `error` set and without tokens; with `raise_on_error` that is a ValueError
+        naming all of them, raised after the others have finished."""
         if return_logits not in (False, True, "none", "last", "all"):
             raise ValueError(f"return_logits must be False, True, 'none', 'last' or 'all', not {return_logits!r}")
         keep_all = return_logits == "all"
@@ -104,15 +131,24 @@ class Engine:
                 raise ValueError(f"request {i}: input_length {r.input_length} != len(input_ids) {len(ids)}")
             gen.append(GenerationRequest(req_id=i, prompt=ids, max_new_tokens=int(r.max_new_tokens),
                                          temperature=float(t), keep_logits=keep_last, keep_all_logits=keep_all))
-        sched = Scheduler(self.runner, self.sampler, self.cfg, eos_token_ids=None)
-        done = sched.run(gen)
+        sched = Scheduler(self.runner, self.sampler, self.cfg, eos_token_ids=self.stop_ids(stop_token_ids))
+        try:
+            done = sched.run(gen)
+        except BaseException:
+            # a step failed: give back what this call's requests hold, so that the engine can go on
+            sched.abort()
+            raise
         out = []
         for r, g in zip(requests, done):
             out.append(Request(input_ids=r.input_ids, input_length=r.input_length,
                                max_new_tokens=r.max_new_tokens,
                                generated_tokens=torch.tensor(g.generated, dtype=torch.long),
                                logits=(torch.stack(g.logit_rows) if keep_all and g.logit_rows
-                                       else g.last_logits if keep_last else None)))
+                                       else g.last_logits if keep_last else None),
+                               error=g.error))
+        failed = [(i, o.error) for i, o in enumerate(out) if o.error]
+        if failed and raise_on_error:
+            raise ValueError("requests that could not run: " + "; ".join(f"request {i}: {e}" for i, e in failed))
         return out
 
 
@@ -129,6 +165,8 @@ def load_model(model_name: str, device: str = "cuda", dtype=torch.bfloat16, **en
 
 
 def generate(model: Engine, requests: Sequence[Request], temperature: float = 0.0,
-             return_logits: Union[bool, str] = False) -> List[Request]:
-    """serve/run.py:238-308."""
-    return model.generate(requests, temperature=temperature, return_logits=return_logits)
+             return_logits: Union[bool, str] = False, stop_token_ids=None,
+             raise_on_error: bool = False) -> List[Request]:
+    """serve/run.py:238-308; `stop_token_ids` and `raise_on_error` as in `Engine.generate`."""
+    return model.generate(requests, temperature=temperature, return_logits=return_logits,
+                          stop_token_ids=stop_token_ids, raise_on_error=raise_on_error)

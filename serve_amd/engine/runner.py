@@ -85,7 +85,7 @@ class ModelRunner:
         creq = model.cache_requests()
         sreq = model.state_requests()
         self.windows = group_windows(creq)
-        per_page = bytes_per_page(creq, self.windows, cfg.page_size, torch.empty((), dtype=rt.dtype).element_size())
+        per_page = bytes_per_page(creq, self.windows, cfg.page_size, rt.dtype)
         if cfg.num_pages is not None:
             num_pages = [int(cfg.num_pages)] * len(self.windows)
         else:
@@ -100,6 +100,7 @@ class ModelRunner:
                                   cfg.max_pages_per_request)
         self.storage = CacheStorage(rt, creq, sreq, self.windows, num_pages, cfg.page_size, cfg.max_requests)
         self._graphs = {}
+        self._graph_pool = None
         # tokens sampled by the latest decode launch, by row: the next launch may read them here
         self.sampled = torch.zeros(max(GRAPH_BATCHES[-1], cfg.max_requests), dtype=torch.int32, device=rt.device)
         self._row_of = {}
@@ -119,6 +120,10 @@ class ModelRunner:
 
     def release(self, req_id) -> None:
         self.cache.release(req_id)
+
+    def forget_launches(self) -> None:
+        """Drop what is remembered of steps launched ahead of the host (after a failed run)."""
+        self._row_of = {}
 
     # -- the step ---------------------------------------------------------------------------------
     @torch.inference_mode()
@@ -155,12 +160,14 @@ class ModelRunner:
         device.  Returns (entry, logits, context lengths)."""
         B = len(segments)
         b_pad = next(b for b in GRAPH_BATCHES if b >= B)
-        mp = self.cfg.max_pages_per_request
+        longest = 1 + max(self.cache.tokens_of(s.req_id) for s in segments)
+        bucket = 256
+        while bucket < longest:
+            bucket *= 2
+        # the block tables of a shape are as wide as its bucket of contexts needs, no wider
+        mp = min(self.cfg.max_pages_per_request, -(-bucket // self.cfg.page_size))
         lay, host, facts = plan_step(segments, self.cache, self.vocab_size, pad_segments_to=b_pad,
                                      fixed_max_pages=mp)
-        bucket = 256
-        while bucket < facts["max_ctx_len"]:
-            bucket *= 2
         key = (b_pad, bucket)
         entry = self._graphs.get(key)
         if entry is None:
@@ -202,9 +209,13 @@ class ModelRunner:
             logits = run()
             if entry.runs >= 2:
                 # every library is loaded and warm by now: capture for the following steps
+                # all graphs take their intermediate buffers from one pool (they never run side by
+                # side); what a graph keeps for itself is its logits [b_pad, V]
+                if self._graph_pool is None:
+                    self._graph_pool = torch.cuda.graph_pool_handle()
                 g = torch.cuda.CUDAGraph()
                 torch.cuda.synchronize()
-                with torch.cuda.graph(g):
+                with torch.cuda.graph(g, pool=self._graph_pool):
                     entry.logits = run()
                 entry.graph = g
         else:

@@ -253,6 +253,8 @@ class Scheduler:
     def _fit_tokens(self, r: GenerationRequest, free: List[int]) -> int:
         """Most tokens of r that the free pages can take now."""
         have = self.cache.tokens_of(r.req_id)
+        if not free:                          # a model without paged cache: pages never bound a portion
+            return r.pending()
         room = min(free) * self.cache.page_size + (-have) % self.cache.page_size
         return room
 
@@ -371,6 +373,23 @@ class Scheduler:
         if self._inflight is not None:
             self._read_back(self._inflight)
             self._inflight = None
+
+    def abort(self) -> None:
+        """Give back the slots and pages of every request that is still running and forget the
+        step in flight: after a step has raised, so that the runner and its cache can be used on."""
+        self._inflight = None
+        for r in list(self.running):
+            if r.req_id in self.cache:
+                self.runner.release(r.req_id)
+            res = self._reservation.pop(r.req_id, None)
+            if res is not None:
+                for g, n in enumerate(res):
+                    self._reserved[g] -= n
+        self.running.clear()
+        self.waiting.clear()
+        forget = getattr(self.runner, "forget_launches", None)
+        if forget is not None:
+            forget()
 
     def run(self, requests: Sequence[GenerationRequest]) -> List[GenerationRequest]:
         """Generate for all requests; returns them in the order given."""

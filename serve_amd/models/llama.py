@@ -25,8 +25,8 @@ def build_llama_spec(cfg: LlamaConfig) -> ModelSpec:
     layers = []
     for i in range(cfg.num_hidden_layers):
         p = f"model.layers.{i}."
-        layers.append(LayerSpec(
-            mixer=PartSpec("gqa_attention", {
+        layers.append(LayerSpec(parts={
+            "mixer": PartSpec("gqa_attention", {
                 "hidden_size": cfg.hidden_size,
                 "num_heads": cfg.num_attention_heads,
                 "num_kv_heads": cfg.num_key_value_heads,
@@ -35,10 +35,10 @@ def build_llama_spec(cfg: LlamaConfig) -> ModelSpec:
                 "window": None,
                 "position": position,
             }),
-            ffn=PartSpec("swiglu", {"hidden_size": cfg.hidden_size,
-                                    "intermediate_size": cfg.intermediate_size}),
-            mixer_norm=norm,
-            ffn_norm=norm,
+            "ffn": PartSpec("swiglu", {"hidden_size": cfg.hidden_size,
+                                       "intermediate_size": cfg.intermediate_size}),
+            "mixer_norm": norm,
+            "ffn_norm": norm},
             weights={
                 "mixer.q_proj.weight": p + "self_attn.q_proj.weight",
                 "mixer.k_proj.weight": p + "self_attn.k_proj.weight",
@@ -63,8 +63,9 @@ def build_llama_spec(cfg: LlamaConfig) -> ModelSpec:
         layers=layers,
         run_order=[RunEntry(layer=i, cache=i) for i in range(cfg.num_hidden_layers)],
         final_norm=norm,
+        # tied, or a checkpoint without lm_head.weight: the head shares the embedding table
         lm_head=PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size,
-                                         "tied": cfg.tie_word_embeddings}),
+                                         "tied": cfg.tie_word_embeddings, "shares": "embedding.weight"}),
         weights={
             "embedding.weight": "model.embed_tokens.weight",
             "final_norm.weight": "model.norm.weight",

@@ -10,7 +10,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..config.spec import ModelSpec, PartSpec
-from ..parts.base import KVCacheRequest, LayerCache, Part, Runtime, StateRequest
+from ..parts.base import LayerCache, Part, Runtime, StateRequest, TokenCacheRequest
 from ..registry import get_part
 
 
@@ -24,6 +24,8 @@ class WeightRequest:
     shape: Tuple[int, ...]
     init: str
     optional: bool
+    alias_of: Optional[str] = None     # "owner.local_name" of the tensor that serves in its place
+    alias_only: bool = False           # the checkpoint's own copy is never read
 
 
 def _make(role: str, spec: PartSpec):
@@ -37,11 +39,13 @@ class Model:
         self.final_norm = _make("norm", spec.final_norm)
         self.lm_head = _make("lm_head", spec.lm_head)
         self.layers = []
-        for ls in spec.layers:
+        for i, ls in enumerate(spec.layers):
             arrangement = get_part("arrangement", ls.arrangement)
-            self.layers.append(arrangement(mixer=_make("mixer", ls.mixer), ffn=_make("feed_forward", ls.ffn),
-                                           mixer_norm=_make("norm", ls.mixer_norm),
-                                           ffn_norm=_make("norm", ls.ffn_norm)))
+            roles = arrangement.PART_ROLES              # part name -> registry role
+            if set(ls.parts) != set(roles):
+                raise ValueError(f"layer {i}: arrangement {ls.arrangement!r} is built from the parts "
+                                 f"{sorted(roles)}, the spec gives {sorted(ls.parts)}")
+            self.layers.append(arrangement(**{name: _make(roles[name], ps) for name, ps in ls.parts.items()}))
         for e in spec.run_order:
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"run order names layer {e.layer}, the model has {len(self.layers)}")
@@ -65,7 +69,8 @@ class Model:
                 key = prefix + pr.name
                 if key not in names:
                     raise KeyError(f"the spec gives no checkpoint name for {owner}.{pr.name}")
-                out.append(WeightRequest(names[key], owner, pr.name, tuple(pr.shape), pr.init, pr.optional))
+                out.append(WeightRequest(names[key], owner, pr.name, tuple(pr.shape), pr.init, pr.optional,
+                                         pr.alias_of, pr.alias_only))
 
         add("embedding", self.embedding, self.spec.weights, "embedding.")
         for i, (layer, ls) in enumerate(zip(self.layers, self.spec.layers)):
@@ -88,13 +93,18 @@ class Model:
                 raise ValueError(f"cache layer {c} is read but never written")
         self._cache_writer_layer = [writers[c] for c in range(n)]
 
-    def cache_requests(self) -> List[Optional[KVCacheRequest]]:
-        """Per cache layer: what the mixer that writes it needs per token."""
-        return [self.layers[l].mixer.cache_request() for l in self._cache_writer_layer]
+    def _cache_owner(self, layer: int) -> Optional[Part]:
+        return self.layers[layer].cache_owner()
+
+    def cache_requests(self) -> List[Optional[TokenCacheRequest]]:
+        """Per cache layer: what the part that writes it keeps per token."""
+        owners = [self._cache_owner(l) for l in self._cache_writer_layer]
+        return [None if o is None else o.cache_request() for o in owners]
 
     def state_requests(self) -> List[Optional[StateRequest]]:
-        """Per cache layer: the fixed-size per-request state its mixer needs."""
-        return [self.layers[l].mixer.state_request() for l in self._cache_writer_layer]
+        """Per cache layer: the fixed-size per-request state its part needs."""
+        owners = [self._cache_owner(l) for l in self._cache_writer_layer]
+        return [None if o is None else o.state_request() for o in owners]
 
     def graph_safe(self) -> bool:
         """Whether every part only enqueues GPU work, so that a step can be captured into a graph."""
@@ -102,20 +112,28 @@ class Model:
 
     # -- loading ------------------------------------------------------------------------------
     def load(self, tensors_by_owner: Dict[str, Dict[str, torch.Tensor]], rt: Runtime) -> None:
+        """Hand every part its tensors.  A request with `alias_of` that got no tensor of its own
+        receives the named tensor of the other part: the same device memory, no copy."""
         self.rt = rt
+        given = {owner: dict(t) for owner, t in tensors_by_owner.items()}
+        for r in self.weight_requests():
+            if r.alias_of is None or r.local_name in given.get(r.owner, {}):
+                continue
+            other = max((o for o in self._owners() if r.alias_of.startswith(o + ".")), key=len, default="")
+            local = r.alias_of[len(other) + 1:]
+            if local not in given.get(other, {}):
+                raise KeyError(f"{r.owner}.{r.local_name} stands for {r.alias_of}, which was not loaded")
+            t = given[other][local]
+            if tuple(t.shape) != tuple(r.shape):
+                raise ValueError(f"{r.owner}.{r.local_name} {list(r.shape)} cannot share {r.alias_of} {list(t.shape)}")
+            given.setdefault(r.owner, {})[r.local_name] = t
         for owner, part in self._owners().items():
-            part.load(tensors_by_owner.get(owner, {}), rt)
-        if getattr(self.lm_head, "weight", 0) is None:
-            # tied output matrix: share the embedding table, no copy
-            self.lm_head.weight = self.embedding.weight
+            part.load(given.get(owner, {}), rt)
 
     # -- running -------------------------------------------------------------------------------
     def forward(self, ctx, caches: List[LayerCache]) -> torch.Tensor:
         """Run the tokens of one step; return fp32 logits [R, V] at ctx.logit_rows."""
-        if getattr(ctx, "src_row", None) is not None:
-            x = self.embedding.forward(ctx.token_ids, ctx.src_row, ctx.prev_tokens)
-        else:
-            x = self.embedding.forward(ctx.token_ids)
+        x = self.embedding.forward(ctx)
         pending = None
         for e in self.spec.run_order:
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)

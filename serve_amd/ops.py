@@ -358,10 +358,13 @@ def qkv_rope_bf16(a: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, pos
 MFMA_ATTENTION_HEAD_DIMS = tuple(range(16, 129, 16))
 
 
-def mfma_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_stride: int) -> bool:
+def mfma_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_stride: int,
+                             scale: float = 1.0) -> bool:
+    """bf16, head sizes 16..128 in steps of 16, page sizes that are multiples of 4, and a positive
+    score scale (the kernels take row maxima of the raw scores and scale afterwards)."""
     P, Hk, page_size, D = k_pages.shape
     return (q.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and D in MFMA_ATTENTION_HEAD_DIMS
-            and page_size % 4 == 0 and q_row_stride % 8 == 0 and q.data_ptr() % 16 == 0)
+            and page_size % 4 == 0 and q_row_stride % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0.0)
 
 
 def attention_splits(max_q_len: int, num_segments: int, num_kv_heads: int, max_ctx_len: int,
@@ -430,9 +433,9 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
     tokens up to the end of the last of them."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
     P, Hk, page_size, D = k_pages.shape
-    _check(mfma_attention_available(q, k_pages, q_row_stride),
-           f"paged_attention_mfma takes bf16, head sizes {MFMA_ATTENTION_HEAD_DIMS} and page sizes that are "
-           f"multiples of 4; got head size {D}, page size {page_size}")
+    _check(mfma_attention_available(q, k_pages, q_row_stride, scale),
+           f"paged_attention_mfma takes bf16, head sizes {MFMA_ATTENTION_HEAD_DIMS}, page sizes that are "
+           f"multiples of 4 and a positive scale; got head size {D}, page size {page_size}, scale {scale}")
     _check(v_pages.shape == (P, Hk, D, page_size) and v_pages.dtype == torch.bfloat16,
            "v_pages must be bf16 [P, Hk, D, page_size]")
     _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
@@ -506,7 +509,7 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
     """Attention over the paged cache for all tokens of the step described by `ctx`
     (`serve_amd.engine.batch.StepContext`): the matrix-core kernel for bf16 where it takes the
     sizes, else the general fp32-arithmetic kernel."""
-    if mfma_attention_available(q, k_pages, q_row_stride):
+    if mfma_attention_available(q, k_pages, q_row_stride, scale):
         Hk = k_pages.shape[1]
         # (first segment, segments, tokens up to their end, longest portion, longest context)
         for s0, n, t_end, max_q, max_ctx in _attention_launches(ctx):

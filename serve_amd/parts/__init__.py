@@ -1,3 +1,4 @@
 """Parts of a layer.  Importing the package registers the standard kinds."""
-from .base import KVCacheRequest, LayerCache, ParamRequest, Part, Runtime, StateRequest  # noqa: F401
+from .base import (CacheTensor, LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime,  # noqa: F401
+                   StateRequest, TokenCacheRequest, kv_cache_request)
 from . import standard  # noqa: F401

@@ -10,16 +10,19 @@ Roles and what each must offer:
                 residual stream `x` in place and returns the normalised activations in the
                 activation dtype; with `rows` it returns only those rows and leaves x alone.
                 `delta` is [T, d], or fp32 [parts, T, d] partial sums to be added in order.
-* position      owned by a mixer; `apply(...)` as the mixer needs it (the rotary part rotates q
-                and k while k and v are written to the cache).
+* position      owned by a mixer, which asks it either for a rotation it can hand to its fused
+                kernels (`rotary()`) or to encode q and k itself (`apply(q, k, positions)`); it
+                never touches the cache: the mixer stores what it keeps.
 * mixer         `forward(h, ctx, cache, writes_cache) -> delta [T, d]`; may ask for per-token
-                cache (`cache_request`) and for per-request state of fixed size
-                (`state_request`).
+                cache (`cache_request`: a list of tensors per token and a retention rule) and
+                for per-request state of fixed size (`state_request`).
 * feed_forward  `forward(h, ctx) -> delta [T, d]`.
-* embedding     `forward(token_ids) -> x` fp32 [T, d].
+* embedding     `forward(ctx) -> x` fp32 [T, d] from the step's token ids (and whatever else of
+                the step it needs: positions for a learned position table).
 * lm_head       `forward(h) -> logits` fp32 [R, V].
-* arrangement   puts a mixer, a feed-forward and their norms together into a layer:
-                `forward(x, pending, ctx, cache, writes_cache) -> pending`.
+* arrangement   puts named parts together into a layer: `PART_ROLES` (name -> role) says which
+                parts it is built from, `cache_owner()` which of them holds the layer's cache
+                and state, `forward(x, pending, ctx, cache, writes_cache) -> pending` runs it.
 """
 from __future__ import annotations
 
@@ -31,29 +34,72 @@ import torch
 
 @dataclass(frozen=True)
 class ParamRequest:
-    """A tensor a part needs, by its local name."""
+    """A tensor a part needs, by its local name.
+
+    `alias_of` names another part's tensor ("embedding.weight": owner, then its local name) that
+    serves when the checkpoint has none for this request; with `alias_only` the checkpoint's own
+    copy is never read (and the random-weights writer makes none).  The part then receives the
+    other part's tensor itself, not a copy: this is how an output matrix is tied to the
+    embedding table."""
 
     name: str
     shape: Tuple[int, ...]
     # how the random-weights writer fills it: "normal" = N(0, 0.02), "ones_normal" = 1 + N(0, 0.1)
     init: str = "normal"
     optional: bool = False
+    alias_of: Optional[str] = None
+    alias_only: bool = False
 
 
 @dataclass(frozen=True)
-class KVCacheRequest:
-    """Per-token cache a mixer needs in its layer: keys and values of `num_kv_heads` heads of
-    `head_dim`, kept for the whole context (`window=None`) or for the last `window` tokens."""
+class CacheTensor:
+    """One tensor a mixer keeps per cached token: `shape` is what one token holds, and a page
+    of it is that shape with the page's tokens put in as axis `token_axis`: ("k", (Hk, D), 1)
+    gives pages [P, Hk, page_size, D]; ("v", (Hk, D), 2) gives [P, Hk, D, page_size];
+    ("latent", (R,), 0) gives [P, page_size, R].  `dtype` None = the activation dtype."""
 
-    num_kv_heads: int
-    head_dim: int
+    name: str
+    shape: Tuple[int, ...]
+    token_axis: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        if not 0 <= self.token_axis <= len(self.shape):
+            raise ValueError(f"cache tensor {self.name!r}: token_axis {self.token_axis} does not fit shape {self.shape}")
+        s = list(self.shape)
+        s.insert(self.token_axis, page_size)
+        return tuple(s)
+
+    def elements_per_token(self) -> int:
+        n = 1
+        for d in self.shape:
+            n *= int(d)
+        return n
+
+
+@dataclass(frozen=True)
+class TokenCacheRequest:
+    """Per-token cache a mixer needs in its layer: the tensors it keeps for every token, for the
+    whole context (`window=None`) or for the last `window` tokens."""
+
+    tensors: Tuple[CacheTensor, ...]
     window: Optional[int] = None
+
+
+def kv_cache_request(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> TokenCacheRequest:
+    """Keys and values of `num_kv_heads` heads of `head_dim` as the attention kernels read them:
+    keys [P, Hk, page, D] (one head's keys of a page are contiguous rows), values
+    [P, Hk, D, page] (transposed inside the page, so that the matrix-core product P.V reads runs
+    of consecutive keys at a fixed dim)."""
+    return TokenCacheRequest((CacheTensor("k", (num_kv_heads, head_dim), 1),
+                              CacheTensor("v", (num_kv_heads, head_dim), 2)), window)
 
 
 @dataclass(frozen=True)
 class StateRequest:
     """Per-request state of fixed size a mixer needs in its layer: one row of this shape for
-    every live request, zeroed when the request is admitted."""
+    every live request, zeroed when the request is admitted.  Rows of a step that belong to no
+    request (padding of a replayed graph) carry the slot -1: a part must skip them."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
@@ -64,21 +110,35 @@ class LayerCache:
     """What the cache manager hands a mixer for one cache layer."""
 
     group: int = -1                              # index into StepContext.groups, -1 = no paged cache
-    k_pages: Optional[torch.Tensor] = None       # [P, Hk, page_size, D]
-    v_pages: Optional[torch.Tensor] = None       # [P, Hk, D, page_size]
+    pages: Dict[str, torch.Tensor] = None        # CacheTensor.name -> [P, *page_shape]
     page_size: int = 0
     state: Optional[torch.Tensor] = None         # [max_requests, *StateRequest.shape]
+
+    def __post_init__(self):
+        if self.pages is None:
+            self.pages = {}
+
+    @property
+    def k_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("k")
+
+    @property
+    def v_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("v")
 
 
 class Runtime:
     """Device, dtypes and settings shared by all parts of a model."""
 
-    def __init__(self, device: torch.device, dtype: torch.dtype):
+    def __init__(self, device: torch.device, dtype: torch.dtype, max_context: Optional[int] = None):
         if dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"compute dtype must be float32 or bfloat16, got {dtype}")
         self.device = torch.device(device)
         self.dtype = dtype                 # activations and cache
         self.exact = dtype == torch.float32
+        # the longest context a request may reach (None = not known): parts whose kernels hold
+        # only up to some position check it when they are loaded
+        self.max_context = max_context
 
     def empty(self, shape, dtype=None) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
@@ -99,8 +159,33 @@ class Part:
         self.rt = rt
 
     # mixers only
-    def cache_request(self) -> Optional[KVCacheRequest]:
+    def cache_request(self) -> Optional[TokenCacheRequest]:
         return None
 
     def state_request(self) -> Optional[StateRequest]:
         return None
+
+
+@dataclass
+class Rotary:
+    """A rotation of pairs of the first `rot_dim` dims of every head of q and k by
+    position * inv_freq[j], as data: what the attention's fused kernels take."""
+
+    inv_freq: torch.Tensor          # fp32 [rot_dim / 2] on the device
+    rot_dim: int
+    adjacent_pairs: bool            # pair j = (2j, 2j + 1); else (j, j + rot_dim / 2)
+
+
+class PositionPart(Part):
+    """Base of position encodings that act on q and k.  Offer `rotary()` if the encoding is a
+    rotation the kernels know, else `apply`; the default is no encoding at all (the order of
+    tokens then enters through the causal mask alone)."""
+
+    graph_safe = True
+
+    def rotary(self) -> Optional[Rotary]:
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], positions: torch.Tensor) -> None:
+        """Encode in place: q [T, Hq, D] and k [T, Hk, D] (views into the projected rows; k is
+        None for a mixer that reads another layer's cache), positions int32 [T]."""

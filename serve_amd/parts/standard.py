@@ -12,7 +12,8 @@ import torch
 from .. import ops
 from ..config.spec import PartSpec
 from ..registry import get_part, register_part
-from .base import KVCacheRequest, LayerCache, ParamRequest, Part, Runtime
+from .base import (LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime, TokenCacheRequest,
+                   kv_cache_request)
 from .linear import linear
 
 
@@ -68,13 +69,20 @@ def rope_inverse_frequencies(head_dim_rot: int, theta: float, scaling: Optional[
     return out.float()
 
 
-class RotaryPosition(Part):
+# largest angle (position * frequency, in radians) whose sine and cosine the bfloat16 kernels'
+# own argument reduction gives to 1e-6; the float32 kernels use the library's sincosf
+ROTARY_MAX_ANGLE_REDUCED = 4.0e6
+
+
+class RotaryPosition(PositionPart):
     """Rotation of pairs of q and k by position * f_j (serve/model.py:234-244).
 
     `pairing="half"`: pair j is (j, j + rot/2), the row order of checkpoints; the reference
     reaches the same scores by permuting the q/k rows and rotating adjacent pairs
     (serve/hf_utils/convert_hf_checkpoint.py:115-118), which is `pairing="adjacent"`.
-    `rot_dim < head_dim` leaves the remaining dims of every head as they are."""
+    `rot_dim < head_dim` leaves the remaining dims of every head as they are.  The part only
+    says what the rotation is (`rotary()`); the attention's kernels carry it out, fused with
+    the projection or the cache write."""
 
     graph_safe = True
 
@@ -89,28 +97,17 @@ class RotaryPosition(Part):
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
-        self.inv_freq = rope_inverse_frequencies(self.rot_dim, self.theta, self.scaling).to(rt.device)
+        f = rope_inverse_frequencies(self.rot_dim, self.theta, self.scaling)
+        if not rt.exact and rt.max_context is not None:
+            top = float(f.max()) * max(rt.max_context - 1, 0)
+            if top > ROTARY_MAX_ANGLE_REDUCED:
+                raise ValueError(f"a context of {rt.max_context} tokens gives rotation angles up to {top:.3g} rad; "
+                                 f"the bfloat16 kernels hold up to {ROTARY_MAX_ANGLE_REDUCED:.3g} "
+                                 "(use dtype float32, or a shorter max_context)")
+        self._rotary = Rotary(f.to(rt.device), self.rot_dim, self.pairing == "adjacent")
 
-    def project_rotate_store(self, h: torch.Tensor, w_qkv: torch.Tensor, positions: torch.Tensor,
-                             slots: torch.Tensor, cache: LayerCache, num_heads: int,
-                             num_kv_heads: int) -> Optional[torch.Tensor]:
-        """The q/k/v product, the rotation and the cache write as one kernel, where the kernel
-        takes the sizes: returns rotated q [T, Hq D], or None (then the caller does the steps
-        one by one)."""
-        if not ops.qkv_rope_available(h, w_qkv, cache.k_pages, self.head_dim, self.rot_dim,
-                                      self.pairing == "adjacent"):
-            return None
-        q = self.rt.empty((h.shape[0], num_heads * self.head_dim))
-        return ops.qkv_rope_bf16(h, w_qkv, q, positions, self.inv_freq, slots, cache.k_pages, cache.v_pages,
-                                 num_heads, num_kv_heads, self.head_dim, cache.page_size)
-
-    def rotate_and_store(self, qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
-                         cache: Optional[LayerCache], num_heads: int, num_kv_heads: int) -> None:
-        ops.rope_kv_write(qkv, positions, self.inv_freq, slots,
-                          None if slots is None else cache.k_pages,
-                          None if slots is None else cache.v_pages,
-                          num_heads, num_kv_heads, self.head_dim, self.rot_dim,
-                          self.pairing == "adjacent", 0 if cache is None else max(cache.page_size, 1))
+    def rotary(self) -> Rotary:
+        return self._rotary
 
 
 # ---------------------------------------------------------------------------------------------
@@ -131,6 +128,8 @@ class GQAAttention(Part):
         if not isinstance(position, PartSpec):
             position = PartSpec(position["kind"], position["params"])
         self.position = get_part("position", position.kind)(**position.params)
+        # a position part that reads back to the host keeps the whole mixer out of graphs
+        self.graph_safe = bool(getattr(self.position, "graph_safe", False))
 
     def param_requests(self) -> List[ParamRequest]:
         d, D = self.hidden_size, self.head_dim
@@ -139,8 +138,8 @@ class GQAAttention(Part):
                 ParamRequest("v_proj.weight", (self.num_kv_heads * D, d)),
                 ParamRequest("o_proj.weight", (d, self.num_heads * D))]
 
-    def cache_request(self) -> KVCacheRequest:
-        return KVCacheRequest(self.num_kv_heads, self.head_dim, self.window)
+    def cache_request(self) -> TokenCacheRequest:
+        return kv_cache_request(self.num_kv_heads, self.head_dim, self.window)
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
@@ -151,24 +150,40 @@ class GQAAttention(Part):
         self.wq = self.wqkv[: self.num_heads * self.head_dim]
         self.wo = tensors["o_proj.weight"]
         self.position.load({}, rt)
+        self._no_freq = torch.empty(0, dtype=torch.float32, device=rt.device)
+
+    def _project_encode_store(self, h: torch.Tensor, ctx, cache: LayerCache, slots: Optional[torch.Tensor]):
+        """q (with k and v behind it in the same rows when they are stored), encoded by position,
+        k and v written to the token's cache slots.  Returns the rows and their stride."""
+        Hq, Hk, D = self.num_heads, self.num_kv_heads, self.head_dim
+        store = slots is not None
+        rot = self.position.rotary()
+        if (store and rot is not None
+                and ops.qkv_rope_available(h, self.wqkv, cache.k_pages, D, rot.rot_dim, rot.adjacent_pairs)):
+            # few rows: product, rotation and cache write are one kernel; only q comes back
+            q = self.rt.empty((h.shape[0], Hq * D))
+            return ops.qkv_rope_bf16(h, self.wqkv, q, ctx.positions, rot.inv_freq, slots, cache.k_pages,
+                                     cache.v_pages, Hq, Hk, D, cache.page_size)
+        qkv = linear(h, self.wqkv if store else self.wq)
+        if rot is None:
+            # an encoding the kernels do not know: the position part works on q and k itself
+            T = qkv.shape[0]
+            k = qkv[:, Hq * D: (Hq + Hk) * D].view(T, Hk, D) if store else None
+            self.position.apply(qkv[:, : Hq * D].view(T, Hq, D), k, ctx.positions)
+            if not store:
+                return qkv
+            inv_freq, rot_dim, adjacent = self._no_freq, 0, False
+        else:
+            inv_freq, rot_dim, adjacent = rot.inv_freq, rot.rot_dim, rot.adjacent_pairs
+        ops.rope_kv_write(qkv, ctx.positions, inv_freq, slots, cache.k_pages if store else None,
+                          cache.v_pages if store else None, Hq, Hk, D, rot_dim, adjacent,
+                          max(cache.page_size, 1))
+        return qkv
 
     def forward(self, h: torch.Tensor, ctx, cache: LayerCache, writes_cache: bool = True) -> torch.Tensor:
-        T = h.shape[0]
         grp = ctx.groups[cache.group]
-        fused = getattr(self.position, "project_rotate_store", None)
-        qkv = None
-        if writes_cache and fused is not None:
-            qkv = fused(h, self.wqkv, ctx.positions, grp.slots, cache, self.num_heads, self.num_kv_heads)
-        if qkv is not None:
-            pass                                # q alone, rotated; k and v are in the cache
-        elif writes_cache:
-            qkv = linear(h, self.wqkv)
-            self.position.rotate_and_store(qkv, ctx.positions, grp.slots, cache, self.num_heads,
-                                           self.num_kv_heads)
-        else:
-            qkv = linear(h, self.wq)
-            self.position.rotate_and_store(qkv, ctx.positions, None, None, self.num_heads, self.num_kv_heads)
-        attn = self.rt.empty((T, self.num_heads * self.head_dim))
+        qkv = self._project_encode_store(h, ctx, cache, grp.slots if writes_cache else None)
+        attn = self.rt.empty((h.shape[0], self.num_heads * self.head_dim))
         ops.paged_attention(qkv, qkv.shape[1], attn, cache.k_pages, cache.v_pages, grp.block_table, ctx,
                             self.num_heads, self.scale, self.window)
         return linear(attn, self.wo, partial_ok=True)      # the following norm adds the parts
@@ -227,29 +242,35 @@ class TokenEmbedding(Part):
         self.rt = rt
         self.weight = tensors["weight"]
 
-    def forward(self, token_ids: torch.Tensor, src_row: Optional[torch.Tensor] = None,
-                prev: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """`src_row` / `prev`: rows whose token was sampled on the device by an earlier step."""
-        x = self.rt.empty((token_ids.numel(), self.hidden_size), torch.float32)
-        return ops.embed(self.weight, token_ids, x, src_row, prev)
+    def forward(self, ctx) -> torch.Tensor:
+        """The rows of the step's tokens.  `ctx.src_row` / `ctx.prev_tokens` (when set): rows whose
+        token was sampled on the device by an earlier step and never reached the host."""
+        x = self.rt.empty((ctx.token_ids.numel(), self.hidden_size), torch.float32)
+        return ops.embed(self.weight, ctx.token_ids, x, ctx.src_row, ctx.prev_tokens)
 
 
 class LinearHead(Part):
-    """logits = h @ W^T in fp32 (serve/model.py:159,226-231).  A tied head has no tensor of its
-    own: the model hands it the embedding table (serve/hf_utils/convert_hf_checkpoint.py:146-147)."""
+    """logits = h @ W^T in fp32 (serve/model.py:159,226-231).  `shares` names the tensor of another
+    part that serves as W when the checkpoint has none of its own; a `tied` head never reads its
+    own (serve/hf_utils/convert_hf_checkpoint.py:146-147).  It then receives that tensor itself:
+    no second copy of the table exists."""
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False,
+                 shares: Optional[str] = "embedding.weight"):
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+        self.shares = shares
+        if self.tied and not shares:
+            raise ValueError("a tied head needs the name of the tensor it shares")
 
     def param_requests(self) -> List[ParamRequest]:
-        # optional: a checkpoint without it shares the embedding table; a tied one may still carry it
-        return [ParamRequest("weight", (self.vocab_size, self.hidden_size), optional=True)]
+        return [ParamRequest("weight", (self.vocab_size, self.hidden_size), alias_of=self.shares,
+                             alias_only=self.tied)]
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = None if self.tied else tensors.get("weight")
+        self.weight = tensors["weight"]
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return linear(h, self.weight, out_dtype=torch.float32)
@@ -264,8 +285,13 @@ class PreNormResidual:
     The additions are folded into the following norm: `pending` is the output of the previous
     part that has not been added to the residual stream yet; the layer returns its own."""
 
+    PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "ffn_norm": "norm"}
+
     def __init__(self, mixer, ffn, mixer_norm, ffn_norm):
         self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+
+    def cache_owner(self) -> Part:
+        return self.mixer
 
     def parts(self) -> Dict[str, Part]:
         return {"mixer": self.mixer, "ffn": self.ffn, "mixer_norm": self.mixer_norm, "ffn_norm": self.ffn_norm}

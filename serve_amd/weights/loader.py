@@ -57,7 +57,7 @@ def check_against(model: Model, reader) -> List[WeightRequest]:
     missing, wrong, present = [], [], []
     for r in requests:
         if r.checkpoint_name not in reader:
-            if not r.optional:
+            if not r.optional and r.alias_of is None:
                 missing.append(r.checkpoint_name)
             continue
         _, shape = reader.info(r.checkpoint_name)
@@ -77,10 +77,9 @@ def load_weights(model: Model, reader, rt: Runtime) -> None:
     part prepare itself (fused matrices and the like)."""
     present = check_against(model, reader)
     by_owner: Dict[str, Dict[str, torch.Tensor]] = {}
-    tied = bool(model.spec.lm_head.params.get("tied", False))
     for r in present:
-        if r.owner == "lm_head" and tied:
-            continue                    # a tied head uses the embedding table; its own copy is not read
+        if r.alias_only:
+            continue                    # another part's tensor serves (a tied head): its own copy is not read
         t = reader.read(r.checkpoint_name)
         t = t.to(device=rt.device, dtype=device_dtype(t.dtype, rt)).contiguous()
         by_owner.setdefault(r.owner, {})[r.local_name] = t
@@ -101,11 +100,10 @@ def _tensor_seed(seed: int, name: str) -> int:
 
 def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16) -> Iterator[Tuple[str, torch.Tensor]]:
     """One tensor per request, a pure function of (seed, tensor name): matrices N(0, 0.02), norm
-    weights 1 + N(0, 0.1), drawn in fp32 on the CPU and rounded to `dtype`.  A tied output
-    matrix is not produced."""
-    tied = bool(model.spec.lm_head.params.get("tied", False))
+    weights 1 + N(0, 0.1), drawn in fp32 on the CPU and rounded to `dtype`.  A tensor that only
+    stands for another part's (a tied output matrix) is not produced."""
     for r in model.weight_requests():
-        if r.owner == "lm_head" and tied:
+        if r.alias_only:
             continue
         g = torch.Generator(device="cpu")
         g.manual_seed(_tensor_seed(seed, r.checkpoint_name))

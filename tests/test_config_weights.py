@@ -76,8 +76,8 @@ def test_registry(tmp_path):
 def test_spec_is_data():
     spec = get_architecture("LlamaForCausalLM").build_spec(util.TINY_A)
     assert [e.layer for e in spec.run_order] == [0, 1] and [e.cache for e in spec.run_order] == [0, 1]
-    assert spec.layers[0].mixer.kind == "gqa_attention" and spec.layers[1].ffn.kind == "swiglu"
-    assert spec.layers[1].mixer.params["position"].params["theta"] == 10000.0
+    assert spec.layers[0].parts["mixer"].kind == "gqa_attention" and spec.layers[1].parts["ffn"].kind == "swiglu"
+    assert spec.layers[1].parts["mixer"].params["position"].params["theta"] == 10000.0
     m = Model(spec)
     assert len(m.cache_requests()) == 2 and m.state_requests() == [None, None]
 

@@ -374,9 +374,9 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         for i in range(cfg.num_hidden_layers):
             p = f"toy.{i}."
             layers.append(LayerSpec(
-                mixer=PartSpec("running_sum", {"hidden_size": cfg.hidden_size}),
-                ffn=PartSpec("swiglu", {"hidden_size": cfg.hidden_size, "intermediate_size": 48}),
-                mixer_norm=norm, ffn_norm=norm,
+                parts={"mixer": PartSpec("running_sum", {"hidden_size": cfg.hidden_size}),
+                       "ffn": PartSpec("swiglu", {"hidden_size": cfg.hidden_size, "intermediate_size": 48}),
+                       "mixer_norm": norm, "ffn_norm": norm},
                 weights={"mixer.proj.weight": p + "proj", "ffn.gate_proj.weight": p + "gate",
                          "ffn.up_proj.weight": p + "up", "ffn.down_proj.weight": p + "down",
                          "mixer_norm.weight": p + "n1", "ffn_norm.weight": p + "n2"}))
@@ -438,28 +438,19 @@ def test_toy_routed_feed_forward_and_other_position_encoding(tmp_path, dtype):
     from serve_amd.config.spec import LayerSpec, ModelSpec, PartSpec, RunEntry
     from serve_amd.engine.batch import Segment
     from serve_amd.engine.engine import Engine
-    from serve_amd.parts.base import ParamRequest, Part
+    from serve_amd.parts.base import ParamRequest, Part, PositionPart
     from serve_amd.parts.linear import linear
     from serve_amd.weights.loader import write_random_model
     from tests.plain import llama_plain as P
 
     d, Hq, Hk, D, I, E, V, L = 48, 3, 1, 16, 40, 3, 61, 2
 
-    class NoRotation(Part):
-        """Position encoding that leaves q and k as they are; it still has to put k and v into
-        the cache, which is the position part's job in the framework's attention."""
+    class NoRotation(PositionPart):
+        """Position encoding that leaves q and k as they are: the base class's `apply` does
+        nothing, and storing k and v in the cache is the attention's own business."""
 
         def __init__(self, head_dim):
             self.head_dim = head_dim
-
-        def load(self, tensors, rt):
-            self.none = torch.empty(0, dtype=torch.float32, device=rt.device)
-
-        def rotate_and_store(self, qkv, positions, slots, cache, num_heads, num_kv_heads):
-            ops.rope_kv_write(qkv, positions, self.none, slots,
-                              None if slots is None else cache.k_pages, None if slots is None else cache.v_pages,
-                              num_heads, num_kv_heads, self.head_dim, 0, False,
-                              0 if cache is None else cache.page_size)
 
     class TopOneExperts(Part):
         def __init__(self, hidden_size, intermediate_size, num_experts):
@@ -523,7 +514,8 @@ def test_toy_routed_feed_forward_and_other_position_encoding(tmp_path, dtype):
                 for e in range(E):
                     for n in ("gate", "up", "down"):
                         weights[f"ffn.experts.{e}.{n}.weight"] = p + f"e{e}.{n}"
-            layers.append(LayerSpec(mixer=attn, ffn=ffn, mixer_norm=norm, ffn_norm=norm, weights=weights))
+            layers.append(LayerSpec(parts={"mixer": attn, "ffn": ffn, "mixer_norm": norm, "ffn_norm": norm},
+                                    weights=weights))
         return ModelSpec(architecture=cfg.architecture, vocab_size=V, hidden_size=d,
                          embedding=PartSpec("token_embedding", {"vocab_size": V, "hidden_size": d}),
                          layers=layers, run_order=[RunEntry(i, i) for i in range(L)], final_norm=norm,

@@ -105,7 +105,7 @@ class Engine:
 
     def generate(self, requests: Sequence[Request], temperature: Union[float, Sequence[float]] = 0.0,
                  return_logits: Union[bool, str] = False, stop_token_ids=None,
-                 raise_on_error: bool = False) -> List[Request]:
+                 raise_on_error: bool = False, step_log: Optional[list] = None) -> List[Request]:
         """Generate up to `max_new_tokens` tokens for every request; results in the order given
         (serve/run.py:304).  `temperature` 0 is greedy (serve/run.py:56-57); one value for all
         requests as in the reference, or one per request.  `return_logits`: False / "none"; True /
@@ -116,7 +116,8 @@ class Engine:
         ids; a request ends with the first of them it generates, which stays in its tokens.
         A request that cannot run (longer than max_context, larger than the cache, empty) comes
         back with `error` set and without tokens; with `raise_on_error` that is a ValueError
-        naming all of them, raised after the others have finished."""
+        naming all of them, raised after the others have finished.  `step_log`: a list that
+        receives one record per step (requests, their token counts, who was sampled)."""
         if return_logits not in (False, True, "none", "last", "all"):
             raise ValueError(f"return_logits must be False, True, 'none', 'last' or 'all', not {return_logits!r}")
         keep_all = return_logits == "all"
@@ -131,13 +132,17 @@ class Engine:
                 raise ValueError(f"request {i}: input_length {r.input_length} != len(input_ids) {len(ids)}")
             gen.append(GenerationRequest(req_id=i, prompt=ids, max_new_tokens=int(r.max_new_tokens),
                                          temperature=float(t), keep_logits=keep_last, keep_all_logits=keep_all))
-        sched = Scheduler(self.runner, self.sampler, self.cfg, eos_token_ids=self.stop_ids(stop_token_ids))
+        sched = Scheduler(self.runner, self.sampler, self.cfg, eos_token_ids=self.stop_ids(stop_token_ids),
+                          record_steps=step_log is not None)
         try:
             done = sched.run(gen)
         except BaseException:
             # a step failed: give back what this call's requests hold, so that the engine can go on
             sched.abort()
             raise
+        finally:
+            if step_log is not None:
+                step_log.extend(sched.step_log)
         out = []
         for r, g in zip(requests, done):
             out.append(Request(input_ids=r.input_ids, input_length=r.input_length,

@@ -16,7 +16,7 @@ import hashlib
 import json
 import os
 import re
-from typing import Dict, Iterator, List, Tuple
+from typing import Dict, Iterator, List, Optional, Tuple
 
 import torch
 
@@ -98,10 +98,14 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(h[:8], "little") & 0x7FFFFFFFFFFFFFFF
 
 
-def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16) -> Iterator[Tuple[str, torch.Tensor]]:
+def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16,
+                   scales: Optional[Dict[str, float]] = None) -> Iterator[Tuple[str, torch.Tensor]]:
     """One tensor per request, a pure function of (seed, tensor name): matrices N(0, 0.02), norm
     weights 1 + N(0, 0.1), drawn in fp32 on the CPU and rounded to `dtype`.  A tensor that only
-    stands for another part's (a tied output matrix) is not produced."""
+    stands for another part's (a tied output matrix) is not produced.  `scales` maps a regular
+    expression to a factor for the matrices whose checkpoint name it matches (a model whose
+    attention scores are of order one instead of 0.03 needs larger q and k projections)."""
+    rules = [(re.compile(p), float(f)) for p, f in (scales or {}).items()]
     for r in model.weight_requests():
         if r.alias_only:
             continue
@@ -112,21 +116,25 @@ def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16)
             t = 1.0 + 0.1 * t
         elif r.init == "normal":
             t = 0.02 * t
+            for pattern, factor in rules:
+                if pattern.search(r.checkpoint_name):
+                    t = t * factor
         else:
             raise ValueError(f"unknown init rule {r.init!r} for {r.checkpoint_name}")
         yield r.checkpoint_name, t.to(dtype)
 
 
-def write_random_model(folder: str, config, seed: int, dtype: torch.dtype = torch.bfloat16) -> str:
+def write_random_model(folder: str, config, seed: int, dtype: torch.dtype = torch.bfloat16,
+                       scales: Optional[Dict[str, float]] = None) -> str:
     """Write `folder/config.json` and `folder/model.safetensors` with random weights for the
-    given typed configuration (any registered architecture)."""
+    given typed configuration (any registered architecture), stored in `dtype`."""
     from ..registry import get_architecture
     arch = get_architecture(config.architecture)
     model = Model(arch.build_spec(config))
     os.makedirs(folder, exist_ok=True)
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(config.to_hf_dict(), f, indent=2)
-    write_safetensors(os.path.join(folder, "model.safetensors"), random_tensors(model, seed, dtype),
+    write_safetensors(os.path.join(folder, "model.safetensors"), random_tensors(model, seed, dtype, scales),
                       metadata={"format": "pt", "seed": seed})
     return folder
 

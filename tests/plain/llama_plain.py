@@ -1,8 +1,8 @@
 """Plain, slow, cache-free implementation of the dense Llama decoder.
 
-Written from the formulas of the reference (`/root/reference/serve/...`, cited per
-function as file:line).  It runs whole sequences on the CPU, one function per part,
-and shares no code with the `serve_amd` package: the tests compare the engine with it.
+Written from the formulas of the reference (`serve/...`, cited per function as file:line).
+It runs whole sequences on the CPU, one function per part, and shares no code with the
+`serve_amd` package: the tests compare the engine with it.
 
 Conventions.  Weights are taken by their checkpoint names (`model.layers.N.self_attn...`)
 in the checkpoint's own row order.  The reference rotates adjacent pairs (2j, 2j+1) and
@@ -136,9 +136,11 @@ def swiglu(x: Tensor, w_gate: Tensor, w_up: Tensor, w_down: Tensor) -> Tensor:
     return ((g * torch.sigmoid(g)) * u) @ w_down.T
 
 
-def attention_part(x: Tensor, w: Dict[str, Tensor], prefix: str, cfg: dict, positions: Tensor) -> Tensor:
+def attention_part(x: Tensor, w: Dict[str, Tensor], prefix: str, cfg: dict, positions: Tensor,
+                   window: Optional[int] = None) -> Tensor:
     """serve/model.py:103-134 without the cache: project, split into heads, rotate q and k,
-    attend causally, project back."""
+    attend causally, project back.  (`window` is not the reference's: a query then sees only the
+    last `window` keys, itself included; for toy models of the tests.)"""
     Hq = cfg["num_attention_heads"]
     Hk = cfg.get("num_key_value_heads") or Hq
     D = head_dim_of(cfg)
@@ -154,16 +156,17 @@ def attention_part(x: Tensor, w: Dict[str, Tensor], prefix: str, cfg: dict, posi
     table = rope_table(positions, freqs)
     q = apply_rope_adjacent(q, table)
     k = apply_rope_adjacent(k, table)
-    o = causal_attention(q, k, v)
+    o = causal_attention(q, k, v, window)
     return o.reshape(S, Hq * D) @ wo.T
 
 
-def decoder_block(x: Tensor, w: Dict[str, Tensor], layer: int, cfg: dict, positions: Tensor) -> Tensor:
+def decoder_block(x: Tensor, w: Dict[str, Tensor], layer: int, cfg: dict, positions: Tensor,
+                  window: Optional[int] = None) -> Tensor:
     """serve/model.py:146-149: x += attn(norm1(x)); x += mlp(norm2(x))."""
     p = f"model.layers.{layer}."
     eps = cfg.get("rms_norm_eps", 1e-5)
     h = rms_norm(x, w[p + "input_layernorm.weight"].to(x.dtype), eps)
-    x = x + attention_part(h, w, p, cfg, positions)
+    x = x + attention_part(h, w, p, cfg, positions, window)
     h = rms_norm(x, w[p + "post_attention_layernorm.weight"].to(x.dtype), eps)
     x = x + swiglu(h, w[p + "mlp.gate_proj.weight"].to(x.dtype), w[p + "mlp.up_proj.weight"].to(x.dtype),
                    w[p + "mlp.down_proj.weight"].to(x.dtype))
@@ -178,13 +181,15 @@ def lm_head_weight(w: Dict[str, Tensor], cfg: dict) -> Tensor:
     return w["lm_head.weight"]
 
 
-def forward(tokens: Sequence[int], w: Dict[str, Tensor], cfg: dict, dtype=torch.float64) -> Tensor:
-    """serve/model.py:196-231 over one whole sequence: logits at every position, [S, V]."""
+def forward(tokens: Sequence[int], w: Dict[str, Tensor], cfg: dict, dtype=torch.float64,
+            windows: Optional[Sequence[Optional[int]]] = None) -> Tensor:
+    """serve/model.py:196-231 over one whole sequence: logits at every position, [S, V].
+    (`windows`: per layer, for toy models of the tests; the reference has none.)"""
     tok = torch.as_tensor(list(tokens), dtype=torch.long)
     positions = torch.arange(len(tok))
     x = w["model.embed_tokens.weight"].to(dtype)[tok]
     for layer in range(cfg["num_hidden_layers"]):
-        x = decoder_block(x, w, layer, cfg, positions)
+        x = decoder_block(x, w, layer, cfg, positions, None if windows is None else windows[layer])
     x = rms_norm(x, w["model.norm.weight"].to(dtype), cfg.get("rms_norm_eps", 1e-5))
     return x @ lm_head_weight(w, cfg).to(dtype).T
 

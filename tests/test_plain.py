@@ -226,3 +226,66 @@ def test_generate_feeds_back_its_own_tokens():
     for t in out:
         assert t == int(P.forward(seq, w, cfg)[-1].argmax())
         seq.append(t)
+
+
+# ---------------------------------------------------------------------------------------------
+# the configurations the engine is compared on can tell a wrong model from a right one
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["AS", "BS", "CS"])
+def test_sharp_models_show_a_wrong_rotation_scale_or_head_mapping(tmp_path, monkeypatch, name):
+    """The engine's bfloat16 runs are held to atol 2e-2 on logits.  With N(0, 0.02) weights the
+    attention scores are about 0.03 and a model without rotation stays within that bound; on the
+    sharp variants (q and k projections 4 times as wide) leaving out the rotation, leaving out
+    D^-0.5 or mapping query head h to KV head h % Hk each moves the logits by more than five
+    times the bound, so a bfloat16 engine with one of these faults cannot pass."""
+    import random
+
+    from tests import util
+    folder = util.make_folder(tmp_path, name)
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    tokens = util.random_tokens(random.Random(1), 60, cfg["vocab_size"])
+    base = P.forward(tokens, w, cfg)
+    need = 5 * util.TOL["bfloat16"]["atol"]
+    real_rope, real_attention = P.apply_rope_adjacent, P.causal_attention
+
+    monkeypatch.setattr(P, "apply_rope_adjacent", lambda x, table: x)
+    assert (P.forward(tokens, w, cfg) - base).abs().max().item() >= need, "no rotation"
+    monkeypatch.setattr(P, "apply_rope_adjacent", real_rope)
+
+    monkeypatch.setattr(P, "causal_attention", lambda q, k, v, window=None, scale=None: real_attention(q, k, v, window, 1.0))
+    assert (P.forward(tokens, w, cfg) - base).abs().max().item() >= need, "no D^-0.5"
+
+    Hq, Hk = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    if Hk > 1:
+        G = Hq // Hk
+        order = [h // G for h in range(Hq)]
+        wrong = [h % Hk for h in range(Hq)]
+        assert order != wrong
+
+        def interleaved(q, k, v, window=None, scale=None):
+            # every query head gets a KV "group" of its own, chosen by h % Hk instead of h // G
+            kk, vv = k[:, wrong, :], v[:, wrong, :]
+            return real_attention(q, kk, vv, window, scale)
+        monkeypatch.setattr(P, "causal_attention", interleaved)
+        assert (P.forward(tokens, w, cfg) - base).abs().max().item() >= need, "h % Hk"
+    monkeypatch.setattr(P, "causal_attention", real_attention)
+    # and the plain model itself is as before
+    torch.testing.assert_close(P.forward(tokens, w, cfg), base)
+
+
+@pytest.mark.parametrize("name", ["A32", "B32"])
+def test_weights_stored_in_32_bit_differ_from_their_bfloat16_rounding(tmp_path, name):
+    """The float32 engine is held to atol 2e-5 on models whose tensors are stored in float32: an
+    engine that dropped the low 16 bits of a weight on the way would miss that bound, since the
+    plain model on the rounded weights differs from the plain model on the stored ones by far
+    more (serve/utils.py:67-71: the checkpoint is cast to the run's dtype, not to bfloat16)."""
+    import random
+
+    from tests import util
+    folder = util.make_folder(tmp_path, name)
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    assert all(t.dtype == torch.float32 for t in w.values())
+    tokens = util.random_tokens(random.Random(2), 40, cfg["vocab_size"])
+    exact = P.forward(tokens, w, cfg)
+    rounded = P.forward(tokens, {k: t.to(torch.bfloat16).float() for k, t in w.items()}, cfg)
+    assert (exact - rounded).abs().max().item() >= 20 * util.TOL["float32"]["atol"]

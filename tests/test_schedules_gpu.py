@@ -1,0 +1,237 @@
+"""The schedules that serving runs, against the plain implementation: many decoding requests
+beside prompt portions in one step (attention then goes out as two launches, sampled tokens
+are fed back on the device), decode steps of 8, 17 and 64 requests replayed from graphs across
+a bucket of context lengths, stop tokens, requests that cannot run, and a run that fails midway."""
+from __future__ import annotations
+
+import json
+import os
+import random
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests import util
+from tests.plain import llama_plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def make_engine(folder, dtype, **kw):
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine
+    base = dict(dtype=dtype, page_size=8, num_pages=400, max_context=512, max_requests=16,
+                max_tokens_per_step=24, prefill_chunk=16)
+    base.update(kw)
+    return Engine.from_folder(folder, EngineConfig(**base))
+
+
+SEED = 77
+
+
+def check_tokens(folder, prompt, got, dtype, what, temperature=0.0, rid=0):
+    """Every token must be the plain sampler's choice from the plain model's logits given the
+    tokens before it (greedy: the best logit; at a temperature: the best of logit / T - log q with
+    the request's own noise), unless two scores lie within the dtype's error of each other."""
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    margin = 1e-4 if dtype == "float32" else util.TOL[dtype]["atol"] / (temperature or 1.0)
+    seq = list(prompt)
+    for i, t in enumerate(got):
+        score = llama_plain.forward(seq, w, cfg)[-1]
+        if temperature:
+            noise = llama_plain.exponential_noise(SEED, rid, i, score.shape[0]).double()
+            score = score / temperature - noise.log()
+        gap = (score.max() - score[t]).item()
+        assert gap <= margin, f"{what}: token {i} = {t} is {gap:.3g} below the best score"
+        seq.append(t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["AS", "BS", "C"])
+def test_many_decoders_beside_prompt_portions(tmp_path, name, dtype):
+    """Nine short requests are decoding when three long prompts arrive and are taken in portions
+    of at most 16 tokens under a budget of 24 tokens a step: steps hold four and more single
+    tokens in front of a portion.  Requests with an even number draw at temperature 0.8, the
+    others are greedy."""
+    from serve_amd.engine.engine import Request
+    folder = util.make_folder(tmp_path, name)
+    vocab = util.tiny_config(name).vocab_size
+    rng = random.Random(21)
+    prompts = [util.random_tokens(rng, rng.randrange(2, 10), vocab) for _ in range(9)]
+    prompts += [util.random_tokens(rng, n, vocab) for n in (70, 95, 61)]
+    new = [22] * 9 + [7, 5, 9]
+    temps = [0.8 if i % 2 == 0 else 0.0 for i in range(len(prompts))]
+    engine = make_engine(folder, dtype, seed=SEED)
+    log = []
+    out = engine.generate([Request(torch.tensor(p), len(p), n) for p, n in zip(prompts, new)], temperature=temps,
+                          step_log=log)
+    mixed = [s for s in log if sum(c == 1 for c in s["counts"]) >= 4 and max(s["counts"]) > 1
+             and s["counts"][:4] == [1, 1, 1, 1]]
+    assert len(mixed) >= 5, "the schedule never put four decoding requests in front of a prompt portion"
+    assert any(len(s["requests"]) >= 10 for s in log)
+    for i, (p, n, r) in enumerate(zip(prompts, new, out)):
+        assert r.error is None and len(r.generated_tokens) == n
+        check_tokens(folder, p, r.generated_tokens.tolist(), dtype, f"{name} {dtype} request {i}", temps[i], i)
+    assert len({tuple(r.generated_tokens.tolist()) for r in out}) == len(out)
+    engine.runner.cache.check_invariants()
+    assert engine.runner.cache.free_pages(0) == 400 and not engine.runner.cache.live_requests()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,count", [("AS", 8), ("BS", 17), ("CS", 64), ("B32", 5)])
+def test_graph_decode_of_many_requests_across_a_context_bucket(tmp_path, name, count, dtype):
+    """`count` requests are decoded one token a step for 45 steps while their contexts pass 256
+    tokens: the steps are replayed from graphs of the padded batch (8, 32, 64) for the buckets up
+    to 256 and up to 512 keys, and every logit of every step is compared with the plain model."""
+    from serve_amd.engine.batch import Segment
+    folder = util.make_folder(tmp_path, name)
+    vocab = util.tiny_config(name).vocab_size
+    rng = random.Random(22)
+    steps = 45
+    lens = [rng.randrange(222, 252) for _ in range(count)]
+    tokens = [util.random_tokens(rng, n + steps, vocab) for n in lens]
+    engine = make_engine(folder, dtype, page_size=16, num_pages=count * 20, max_requests=max(count, 8),
+                         max_tokens_per_step=4096, prefill_chunk=4096)
+    runner = engine.runner
+    for i in range(count):
+        assert runner.admit(i)
+    for lo in range(0, count, 8):                      # the prompts, eight requests a step
+        engine.step([Segment(i, tokens[i][: lens[i]], []) for i in range(lo, min(count, lo + 8))])
+    got = [[] for _ in range(count)]
+    for s in range(steps):
+        logits = engine.step([Segment(i, [tokens[i][lens[i] + s]], [0]) for i in range(count)])
+        assert logits.shape == (count, vocab)
+        for i in range(count):
+            got[i].append(logits[i])
+    b_pad = next(b for b in (1, 2, 4, 8, 16, 32, 64) if b >= count)
+    for bucket in (256, 512):
+        entry = runner._graphs.get((b_pad, bucket))
+        assert entry is not None and entry.graph is not None, f"no graph was replayed for {(b_pad, bucket)}"
+        assert entry.layout.MP == bucket // 16            # the tables are as wide as the bucket needs
+    for i in range(count):
+        want = util.plain_logits(folder, tokens[i])[lens[i]:]
+        util.assert_close(torch.stack(got[i]), want, dtype, f"{name} {dtype} request {i} of {count}")
+        runner.release(i)
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stop_tokens_end_a_request_and_free_its_pages(tmp_path, dtype):
+    """A token id that the greedy continuation of request 1 contains ends it there (the id stays
+    in its tokens); requests whose continuation does not contain it are unchanged; its pages and
+    slot are free from that step on; with stop tokens no step is launched ahead of the host."""
+    from serve_amd.engine.engine import Request, generate, load_model
+    folder = util.make_folder(tmp_path, "AS")           # untied head: its greedy continuations vary
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    rng = random.Random(23)
+    prompts = [util.random_tokens(rng, n, 256) for n in (6, 11, 3, 19)]
+    full = [llama_plain.generate(p, 12, w, cfg) for p in prompts]
+    # the first token of request 1's continuation, from its third on, that it has not generated before
+    at = next(j for j in range(2, 12) if full[1][j] not in full[1][:j])
+    stop = full[1][at]
+
+    def cut(seq):
+        return seq[: seq.index(stop) + 1] if stop in seq else seq
+    engine = load_model(folder, "cuda", dtype, page_size=4, num_pages=40, max_context=64, max_requests=4,
+                        max_tokens_per_step=16, prefill_chunk=8)
+    log = []
+    out = engine.generate([Request(torch.tensor(p), len(p), 12) for p in prompts], stop_token_ids=[stop],
+                          step_log=log)
+    for i, (p, r) in enumerate(zip(prompts, out)):
+        got = r.generated_tokens.tolist()
+        if dtype == "float32":
+            assert got == cut(full[i]), f"request {i}"
+        else:
+            check_tokens(folder, p, got, dtype, f"request {i} with a stop token")
+            assert stop not in got[:-1] and (len(got) == 12 or got[-1] == stop)
+    if dtype == "float32":
+        assert len(out[1].generated_tokens) == at + 1
+        last = max(i for i, s in enumerate(log) if 1 in s["requests"])
+        assert 1 in log[last]["sampled"] and any(0 in s["requests"] or 3 in s["requests"] for s in log[last + 1:])
+    runner = engine.runner
+    assert runner._eager_launches == 0 and all(e.launches == 0 for e in runner._graphs.values())
+    runner.cache.check_invariants()
+    assert runner.cache.free_pages(0) == 40 and runner.cache.free_slots() == 4
+    # without stop tokens (the default, and the reference's behaviour) every request runs to its end
+    plain_out = generate(engine, [Request(torch.tensor(p), len(p), 12) for p in prompts])
+    assert all(len(r.generated_tokens) == 12 for r in plain_out)
+    # "eos" takes the ids from the configuration, which this model folder does not name
+    with pytest.raises(ValueError, match="eos_token_id"):
+        engine.generate([Request(torch.tensor(prompts[0]), 6, 2)], stop_token_ids="eos")
+
+
+def test_command_line_stops_at_the_given_token(tmp_path):
+    folder = util.make_folder(tmp_path, "AS")
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    prompt = util.random_tokens(random.Random(24), 9, 256)
+    full = llama_plain.generate(prompt, 10, w, cfg)
+    stop = next(t for j, t in enumerate(full) if j >= 2 and t not in full[:j])
+    want = full[: full.index(stop) + 1]
+    ids = tmp_path / "prompts.txt"
+    ids.write_text(json.dumps(prompt) + "\n")
+    proc = subprocess.run([sys.executable, "-m", "serve_amd", "generate", "--model", folder, "--dtype", "float32",
+                           "--prompt-ids", str(ids), "--max-new-tokens", "10", "--stop-token-ids", str(stop),
+                           "--num-pages", "16", "--page-size", "8", "--max-context", "64", "--max-requests", "2"],
+                          capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert json.loads(proc.stdout.strip().splitlines()[-1]) == want
+
+
+def test_requests_that_cannot_run_come_back_with_an_error(tmp_path):
+    """A prompt longer than max_context beside a good request, through the entry point: the good
+    one is generated, the other says why it was not; `raise_on_error` makes that an exception."""
+    from serve_amd.engine.engine import Request, generate, load_model
+    folder = util.make_folder(tmp_path, "A")
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    engine = load_model(folder, "cuda", torch.float32, page_size=4, num_pages=32, max_context=64, max_requests=4)
+    good = [5, 9, 200, 31]
+    reqs = [Request(torch.tensor([1] * 80), 80, 4), Request(torch.tensor(good), 4, 6),
+            Request(torch.tensor([], dtype=torch.long), 0, 3)]
+    out = generate(engine, reqs)
+    assert "max_context" in out[0].error and len(out[0].generated_tokens) == 0
+    assert out[1].error is None and out[1].generated_tokens.tolist() == llama_plain.generate(good, 6, w, cfg)
+    assert "empty" in out[2].error
+    with pytest.raises(ValueError, match="request 0.*max_context"):
+        generate(engine, reqs, raise_on_error=True)
+    engine.runner.cache.check_invariants()
+    assert not engine.runner.cache.live_requests()
+
+
+def test_a_run_that_fails_midway_gives_everything_back(tmp_path):
+    """A step raises in the middle of `generate`: the requests' slots and pages are given back, and
+    the same engine generates the same requests afterwards."""
+    from serve_amd.engine.engine import Request
+    folder = util.make_folder(tmp_path, "A")
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    engine = make_engine(folder, "float32", page_size=4, num_pages=60, max_context=64, max_requests=4,
+                         max_tokens_per_step=8, prefill_chunk=8)
+    rng = random.Random(25)
+    prompts = [util.random_tokens(rng, n, 256) for n in (12, 5, 9)]
+    reqs = [Request(torch.tensor(p), len(p), 6) for p in prompts]
+    runner = engine.runner
+    real = {name: getattr(runner, name) for name in ("step", "step_launch", "decode_launch")}
+    calls = {"n": 0}
+
+    def failing(name):
+        def f(*a, **k):
+            calls["n"] += 1
+            if calls["n"] == 4:
+                raise RuntimeError("a step failed")
+            return real[name](*a, **k)
+        return f
+    for name in real:
+        setattr(runner, name, failing(name))
+    with pytest.raises(RuntimeError, match="a step failed"):
+        engine.generate(reqs)
+    for name, fn in real.items():
+        setattr(runner, name, fn)
+    runner.cache.check_invariants()
+    assert not runner.cache.live_requests() and runner.cache.free_pages(0) == 60
+    out = engine.generate(reqs)
+    for p, r in zip(prompts, out):
+        assert r.generated_tokens.tolist() == llama_plain.generate(p, 6, w, cfg)

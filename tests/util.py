@@ -47,11 +47,27 @@ TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 TOL = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=2e-2, rtol=2e-2)}
 
 
+# q and k projections of the "sharp" variants are drawn 4 times as wide: attention scores are of
+# order one instead of 0.03, softmax picks keys instead of averaging them, and a fault in
+# the rotation, the score scale or the head mapping moves the logits by far more than the
+# bfloat16 bound (tests/test_plain.py asserts that it does)
+SHARP_SCALES = {r"self_attn\.(q|k)_proj": 4.0}
+
+
+def tiny_config(name: str):
+    """name = A, B or C, then S for the sharp variant, then 32 for tensors stored in float32."""
+    return TINY[name[0]][0]
+
+
 def make_folder(tmp_path, name: str) -> str:
-    cfg, seed = TINY[name]
+    cfg, seed = TINY[name[0]]
+    rest = name[1:]
+    sharp = rest.startswith("S")
+    stored = torch.float32 if rest.endswith("32") else torch.bfloat16
+    assert rest in ("", "S", "32", "S32"), name
     folder = os.path.join(str(tmp_path), f"tiny_{name}")
     if not os.path.isdir(folder):
-        write_random_model(folder, cfg, seed)
+        write_random_model(folder, cfg, seed, dtype=stored, scales=SHARP_SCALES if sharp else None)
     return folder
 
 

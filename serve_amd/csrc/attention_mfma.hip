@@ -1043,7 +1043,18 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
 
 extern "C" int sa_attention_mfma_head_dim() { return HD; }
 
-constexpr int COMPUTE_UNITS = 256;
+// compute units of the current device (asked once per device; 256 if the runtime will not say)
+static int compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
 
 // A step whose segments have at most 16 rows each (single decoded tokens) takes the one-wave kernel,
 // any other the prompt kernel.  `in_workgroup` (such steps only, num_splits 1): the key range of every
@@ -1106,7 +1117,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
     const long long rows = (long long)max_q_len * G;
     const int kw = rows > 64 ? 2 : 4;
     const long long groups = (rows + 256 / kw - 1) / (256 / kw);
-    const int pair = num_splits == 1 && (groups + 1) / 2 * Hk * B >= COMPUTE_UNITS;
+    const int pair = num_splits == 1 && (groups + 1) / 2 * Hk * B >= compute_units();
     const long long items = pair ? (groups + 1) / 2 : groups;
     if (items * Hk > 0x7fffffffLL || (long long)Hk * page_size * HD * 2 > 0x7fffffffLL) return SA_ERR_ARG;
     dim3 grid((unsigned)(items * Hk), B * num_splits);

@@ -69,11 +69,13 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
-// sin and cos of an angle of up to about 2e5 rad (a position times a frequency of at most 1), to
-// about 1e-6: the library's sincosf spends over a thousand cycles on arguments this large.  The
-// multiple of 2 pi is taken off in three steps whose constants have few enough bits for the first
-// products to be exact (6.28125 = 201/32; 2029/2^20; the rest), the remainder goes to the
-// hardware's sine and cosine, which take their argument in turns.
+// sin and cos of an angle of up to 4e6 rad (a position times a frequency of at most 1), to about
+// 1e-6: the library's sincosf spends over a thousand cycles on arguments this large.  The multiple
+// of 2 pi is taken off in three steps whose constants have few enough bits for the first two
+// remainders to be exact (6.28125 = 201/32; 2029/2^20; the rest: with k < 2^20 the first remainder
+// is a multiple of 2^-5 below 2^11, the second a multiple of 2^-20 below 4), the last remainder
+// goes to the hardware's sine and cosine, which take their argument in turns.  Callers keep their
+// angles within the bound (the rotary part refuses longer contexts when it is loaded).
 __device__ __forceinline__ void sincos_reduced(float x, float* sn, float* cs) {
   const float k = rintf(x * 0.15915494309189535f);
   float r = fmaf(-k, 6.28125f, x);

@@ -11,6 +11,9 @@ among the entry's tokens whose logits are written; `end` lists requests that are
 the step, whose pages and slot are given back.  A request is admitted when it first appears.
 For a step in which something is wanted `<out>/<step>.f32` holds the logits at the wanted
 places, in the order of the entries and of `want`, little-endian fp32 [wanted, vocab].
+For every step with entries `<out>/<step>.pages.json` holds, per entry, the page ids its
+request holds after the step, one list per cache group in the order of the request's tokens
+(-1: a page that a window has passed and that was given back).
 After every step `done <step>` is printed and flushed.
 """
 from __future__ import annotations
@@ -69,6 +72,13 @@ def run_trace(engine: Engine, lines: Iterable[str], out_dir: str, log: Optional[
                 tmp = os.path.join(out_dir, f".{step}.f32.tmp")
                 arr.tofile(tmp)
                 os.replace(tmp, os.path.join(out_dir, f"{step}.f32"))
+            cache = runner.cache
+            pages = {str(s.req_id): [list(cache.block_table(s.req_id, g)) for g in range(cache.num_groups)]
+                     for s in segments}
+            tmp = os.path.join(out_dir, f".{step}.pages.tmp")
+            with open(tmp, "w") as f:
+                json.dump(pages, f)
+            os.replace(tmp, os.path.join(out_dir, f"{step}.pages.json"))
         for rid in rec.get("end", []):
             if rid in runner.cache:
                 runner.release(rid)

@@ -69,6 +69,20 @@ def _ret(code: int, what: str) -> None:
         raise KernelError(f"{what}: {reason}")
 
 
+_CU_COUNT = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the device (asked once): the launch policies below fill these."""
+    if not torch.cuda.is_available():
+        return 256                      # planning on a host without a GPU (tests of the policies)
+    dev = torch.cuda.current_device() if device is None else torch.device(device).index or 0
+    n = _CU_COUNT.get(dev)
+    if n is None:
+        n = _CU_COUNT[dev] = int(torch.cuda.get_device_properties(dev).multi_processor_count)
+    return n
+
+
 def _i32(t: torch.Tensor, n: int, name: str) -> None:
     _check(t.dtype == torch.int32 and t.numel() >= n, f"{name} must be int32 with at least {n} entries")
 
@@ -278,18 +292,19 @@ def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tor
 def split_k_parts(M: int, N: int, K: int) -> int:
     """Into how many slices the inner dimension of a few-row product is cut across workgroups so
     that a matrix with few rows still fills the chip: 1 means no cut.  One or two rows: a workgroup
-    takes 16 weight rows (about 1024 workgroups wanted, slices of at least 256); from three rows on
+    takes 16 weight rows (about four workgroups per compute unit wanted, slices of at least 256); from three rows on
     it takes 32 (one workgroup per compute unit wanted, slices of at least 512)."""
     if N >= 8192:
         return 1
+    cus = compute_units()
     parts = 1
     if M > 2:
         groups = -(-N // 32)
-        while parts < 8 and groups * parts < 256 and K // (parts * 2) >= 512:
+        while parts < 8 and groups * parts < cus and K // (parts * 2) >= 512:
             parts *= 2
         return parts
     tiles = -(-N // 16)
-    while parts < 4 and tiles * parts < 1024 and K // (parts * 2) >= 512:
+    while parts < 4 and tiles * parts < 4 * cus and K // (parts * 2) >= 512:
         parts *= 2
     return parts
 
@@ -370,7 +385,7 @@ def mfma_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_strid
 def attention_splits(max_q_len: int, num_segments: int, num_kv_heads: int, max_ctx_len: int,
                      group_size: int = 1) -> int:
     """Into how many parts the key range of a launch is cut so that the chip is filled.
-    Single decoded tokens: about 512 waves in all (more cost more in the merge than they gain), and
+    Single decoded tokens: about two waves per compute unit in all (more cost more in the merge than they gain), and
     no part shorter than 64 keys.  Prompt portions that are at most a quarter of their context (a
     long prompt taken in portions): about one workgroup of 128 rows per compute unit, parts of at
     least 1024 keys; portions that are most of their context are never cut, the causal mask makes
@@ -381,7 +396,7 @@ def attention_splits(max_q_len: int, num_segments: int, num_kv_heads: int, max_c
         groups = -(-max_q_len * group_size // 128)
         workgroups = groups * num_kv_heads * num_segments
         splits = 1
-        while splits < 8 and workgroups * splits < 256 and max_ctx_len // (splits * 2) >= 1024:
+        while splits < 8 and workgroups * splits < compute_units() and max_ctx_len // (splits * 2) >= 1024:
             splits *= 2
         return splits
     # both inputs are rounded up to powers of two, so that a step run eagerly and the same step
@@ -393,7 +408,7 @@ def attention_splits(max_q_len: int, num_segments: int, num_kv_heads: int, max_c
     while segs < num_segments:
         segs *= 2
     by_length = max(1, ctx // 64)
-    by_waves = max(1, 512 // (segs * num_kv_heads))
+    by_waves = max(1, 2 * compute_units() // (segs * num_kv_heads))
     return max(1, min(by_length, by_waves, 64))
 
 

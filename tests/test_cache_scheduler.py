@@ -131,11 +131,18 @@ def test_plan_step_arrays():
     lay, host, facts = plan_step([Segment("a", [9, 9], [])], cm, 100)
     assert v(lay.positions, 2) == [5, 6] and v(lay.slots[0], 2) == [ta[1] * 4 + 1, ta[1] * 4 + 2]
     assert facts["ctx_lens"] == [7] and lay.R == 0
+    # padding rows of a step of fixed shape belong to no request: no cache slot, no state slot
+    for segs in ([Segment("b", [8], [0])], [Segment("b", [8, 8], []), Segment("a", [3], [0])]):
+        lay, host, facts = plan_step(segs, cm, 100, pad_segments_to=4)
+        n = len(segs)
+        assert v(lay.state_slots, 4)[:n] == [cm.slot_of(s.req_id) for s in segs]
+        assert v(lay.state_slots, 4)[n:] == [-1] * (4 - n)
+        assert v(lay.slots[0], lay.T)[-(4 - n):] == [-1] * (4 - n) and v(lay.ctx_len, 4)[n:] == [1] * (4 - n)
     # refusals leave everything as it was
     free = cm.free_pages()
     with pytest.raises(OutOfPages):
         plan_step([Segment("a", [1] * 20, []), Segment("b", [1] * 20, [])], cm, 100)
-    assert cm.free_pages() == free and cm.tokens_of("a") == 7
+    assert cm.free_pages() == free and cm.tokens_of("a") == 8
     with pytest.raises(ValueError, match="vocabulary"):
         plan_step([Segment("a", [100], [])], cm, 100)
     with pytest.raises(ValueError, match="twice"):

@@ -263,3 +263,17 @@ def test_attention_launch_policy_is_the_same_for_a_step_and_its_graph_replay():
             bucket *= 2
         assert ops.attention_splits(1, B, Hk, ctx, G) == ops.attention_splits(1, b_pad, Hk, bucket, G)
         assert ops.attention_in_workgroup(1, B, ctx, G) == ops.attention_in_workgroup(1, b_pad, bucket, G)
+
+
+def test_rotary_part_refuses_contexts_beyond_its_kernels_angles():
+    """The bfloat16 kernels reduce the rotation angle themselves and hold up to 4e6 rad: a
+    longer context is refused when the part is loaded, not rotated wrongly (float32 has no limit)."""
+    import pytest
+    from serve_amd.parts.base import Runtime
+    from serve_amd.parts.standard import RotaryPosition
+    part = RotaryPosition(head_dim=64, rot_dim=64, theta=500000.0)
+    with pytest.raises(ValueError, match="rotation angles"):
+        part.load({}, Runtime(torch.device("cpu"), torch.bfloat16, max_context=8_000_000))
+    part.load({}, Runtime(torch.device("cpu"), torch.bfloat16, max_context=1_000_000))
+    part.load({}, Runtime(torch.device("cpu"), torch.float32, max_context=8_000_000))
+    assert part.rotary().rot_dim == 64 and not part.rotary().adjacent_pairs

@@ -160,6 +160,34 @@ def test_rope_kv_write_of_many_tokens(T, Hq, Hk, D, ps):
     assert v_pages.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rope_at_far_positions(dtype):
+    """Positions up to four million with a highest frequency of 1 rad a token: the angle is a
+    32-bit product of millions of radians, and its sine and cosine must still be those of that
+    product (the bfloat16 kernels reduce the argument themselves; `RotaryPosition` refuses
+    contexts whose angles go beyond what this test covers)."""
+    from serve_amd import ops
+    from serve_amd.parts.standard import ROTARY_MAX_ANGLE_REDUCED
+    Hq, Hk, D, ps = 2, 1, 32, 4
+    pos = torch.tensor([199_999, 200_001, 524_287, 1_000_000, 1_048_577, 2_500_003, 3_999_999, 3_141_593],
+                       dtype=torch.int32, device=DEV)
+    assert pos.max().item() < ROTARY_MAX_ANGLE_REDUCED <= 4.0e6
+    T = pos.numel()
+    qkv = rnd((T, (Hq + 2 * Hk) * D), DT[dtype], 26)
+    qkv0 = qkv.clone()
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+    assert inv_freq[0].item() == 1.0
+    slots = torch.arange(T, dtype=torch.int32, device=DEV)
+    k_pages = torch.zeros((2, Hk, ps, D), dtype=DT[dtype], device=DEV)
+    v_pages = torch.zeros((2, Hk, D, ps), dtype=DT[dtype], device=DEV)
+    ops.rope_kv_write(qkv, pos, inv_freq, slots, k_pages, v_pages, Hq, Hk, D, D, False, ps)
+    x = qkv0.double().view(T, Hq + 2 * Hk, D)
+    t = dict(atol=2e-5, rtol=1e-5) if dtype == "float32" else tol(dtype)
+    torch.testing.assert_close(qkv.double().view(T, -1, D)[:, :Hq], rope_ref(x[:, :Hq], pos, inv_freq, D, False), **t)
+    page, off = (slots // ps).long(), (slots % ps).long()
+    torch.testing.assert_close(k_pages.double()[page, :, off, :], rope_ref(x[:, Hq:Hq + Hk], pos, inv_freq, D, False), **t)
+
+
 def test_rope_depends_on_distance_only():
     """<rope(q, m), rope(k, n)> depends on m - n: shift all positions and compare the scores."""
     from serve_amd import ops

@@ -64,29 +64,45 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
     return [[rng.randrange(vocab) for _ in range(length)] for _ in range(n)]
 
 
+def head_start(engine, batch: int, prompt_len: int) -> int:
+    """An upper bound of the steps that the prompts of `batch` requests take: the requests whose
+    prompts are done first decode that many tokens before the last one joins them."""
+    per_step = max(1, min(engine.cfg.prefill_chunk, engine.cfg.max_tokens_per_step - batch))
+    return batch * (-(-prompt_len // per_step))
+
+
 def decode_run(engine, batch: int, prompt_len: int, warmup: int, steps: int, seed: int):
-    """Prefill `batch` prompts, run `warmup` untimed and `steps` timed decode steps.
-    Returns (seconds, mean context during the timed steps)."""
+    """Prefill `batch` prompts, run `warmup` untimed and `steps` timed decode steps in which every
+    one of the `batch` requests decodes one token (checked from the scheduler's record: a request
+    that ended early would make the later steps cheaper than they are).  Returns (seconds, mean
+    context of the requests during the timed steps)."""
     import torch
     from serve_amd.engine.scheduler import GenerationRequest, Scheduler
     prompts = random_prompts(batch, prompt_len, engine.model.spec.vocab_size, seed)
-    reqs = [GenerationRequest(i, p, warmup + steps + 2) for i, p in enumerate(prompts)]
-    sched = Scheduler(engine.runner, engine.sampler, engine.cfg)
+    # requests whose prompts are done decode while the others' prompts still run: every request gets
+    # enough tokens to stay until the last timed step
+    spare = head_start(engine, batch, prompt_len)
+    reqs = [GenerationRequest(i, p, spare + warmup + steps + 2) for i, p in enumerate(prompts)]
+    sched = Scheduler(engine.runner, engine.sampler, engine.cfg, record_steps=True)
     sched.add(reqs)
     while any(r.pending() > 1 or r.fed == 0 for r in reqs):
         assert sched.step()
     for _ in range(warmup):
         assert sched.step()
     torch.cuda.synchronize()
-    ctx0 = reqs[0].fed
+    ctx0 = sum(r.fed for r in reqs) / batch
+    first = len(sched.step_log)
     t0 = time.perf_counter()
     for _ in range(steps):
         sched.step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    assert all(len(r.generated) >= warmup + steps for r in reqs)
-    while sched.step():
-        pass
+    timed = sched.step_log[first:]
+    assert len(timed) == steps and all(len(t["requests"]) == batch and set(t["counts"]) == {1} for t in timed), \
+        "a timed step did not decode one token for every request of the batch"
+    # the rest of their tokens is not needed: end the requests and give their pages back
+    sched.abort()
+    torch.cuda.synchronize()
     return dt, ctx0 + (steps + 1) / 2.0
 
 
@@ -112,55 +128,82 @@ def prefill_run(engine, tokens: int, repeats: int, seed: int):
 
 
 def measured_ceilings():
-    """What the device itself reaches with the library's plain operations: a copy of 1 GiB (bytes
-    read + written per second), a reduction over 1 GiB (bytes read per second), and a square bf16
-    product of 8192 (flops per second)."""
+    """What the device itself reaches: with the package's own plain kernels a read of 2 GiB that
+    keeps nothing and a copy of 2 GiB (serve_amd/csrc/membench.hip), and with the library's
+    operations a copy of 2 GiB (bytes read + written per second), a reduction over 2 GiB (bytes read
+    per second) and a square bf16 product of 8192 (flops per second)."""
     import torch
+
+    from serve_amd import ops
     dev = "cuda:0"
 
-    def best(fn, repeats=5):
+    def best(fn, repeats=3, launches=5):
+        """Seconds per call: the best of `repeats` rounds of `launches` calls between two events."""
+        fn()
         times = []
-        for _ in range(repeats + 1):
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            fn()
+            e0.record()
+            for _ in range(launches):
+                fn()
+            e1.record()
             torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-        return min(times[1:])
+            times.append(e0.elapsed_time(e1) * 1e-3 / launches)
+        return min(times)
 
-    n = 512 * 1024 * 1024
+    n = 1024 * 1024 * 1024                      # 2 GiB, far beyond the caches
     src = torch.ones(n, dtype=torch.bfloat16, device=dev)
     dst = torch.empty_like(src)
     copy = 2 * 2 * n / best(lambda: dst.copy_(src))
     read = 2 * n / best(lambda: torch.sum(src, dtype=torch.float32))
+    grids = [k * ops.compute_units() for k in (2, 32, 256)]     # few long-running workgroups to many short ones
+    own_read = max(2 * n / best(lambda: ops.read_bytes(src, g)) for g in grids)
+    own_copy = max(2 * 2 * n / best(lambda: ops.copy_bytes(dst, src, g)) for g in grids)
     del src, dst
     a = torch.randn(8192, 8192, dtype=torch.bfloat16, device=dev)
     b = torch.randn(8192, 8192, dtype=torch.bfloat16, device=dev)
     c = torch.empty(8192, 8192, dtype=torch.bfloat16, device=dev)
     gemm = 2 * 8192 ** 3 / best(lambda: torch.mm(a, b.t(), out=c))
-    return {"copy": copy, "read": read, "gemm": gemm}
+    return {"copy": copy, "read": read, "gemm": gemm, "own_read": own_read, "own_copy": own_copy}
 
 
-def report(engine, cfg, steps: int, warmup: int) -> int:
+def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
     """`--report`: every number of the measurement with the bytes or flops it stands for, as a
-    share of the published peaks and of the ceilings measured on this device."""
+    share of the published peaks and of the ceilings measured on this device.  With `make_engine`
+    (context -> engine) also decode steps at contexts of 32k and 128k tokens."""
+    import torch
     ceil = measured_ceilings()
-    print(f"measured ceilings: copy {ceil['copy'] / 1e12:.2f} TB/s (read + write), reduction "
-          f"{ceil['read'] / 1e12:.2f} TB/s (read), 8192^3 bf16 product {ceil['gemm'] / 1e15:.3f} PFLOP/s")
-    bw = max(ceil["copy"], ceil["read"])
+    print(f"measured ceilings: own read kernel {ceil['own_read'] / 1e12:.2f} TB/s, own copy kernel "
+          f"{ceil['own_copy'] / 1e12:.2f} TB/s (read + write); library: copy {ceil['copy'] / 1e12:.2f} TB/s "
+          f"(read + write), reduction {ceil['read'] / 1e12:.2f} TB/s (read), 8192^3 bf16 product "
+          f"{ceil['gemm'] / 1e15:.3f} PFLOP/s")
+    bw = max(ceil["copy"], ceil["read"], ceil["own_read"], ceil["own_copy"])
     print(f"{'workload':34s} {'ms/step':>8s} {'tokens/s':>10s} {'GB or TFLOP':>12s} {'achieved':>14s} {'of peak':>8s} "
           f"{'of measured':>11s}")
-    for batch, prompt_len, n in ((1, 256, 250), (8, 256, 250), (64, 256, 250), (8, 4096 - steps - warmup - 3, steps)):
-        dt, mean_ctx = decode_run(engine, batch, prompt_len, warmup if prompt_len > 256 else 4, n, seed=20 + batch)
+
+    def decode_row(eng, batch, prompt_len, w, n):
+        dt, mean_ctx = decode_run(eng, batch, prompt_len, w, n, seed=20 + batch)
         nbytes = weight_bytes(cfg) + batch * mean_ctx * kv_bytes_per_token(cfg)
         rate = nbytes / (dt / n)
         print(f"{f'decode, batch {batch}, context ~{int(mean_ctx)}':34s} {dt / n * 1e3:8.3f} {batch * n / dt:10.0f} "
-              f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}")
+              f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}", flush=True)
+    for batch, prompt_len, n in ((1, 256, 250), (8, 256, 250), (64, 256, 250)):
+        decode_row(engine, batch, prompt_len, 4, n)
+    decode_row(engine, 8, 4096 - steps - warmup - 3 - head_start(engine, 8, 4096), warmup, steps)
     T = 2048
     pt = prefill_run(engine, T, repeats=5, seed=7)
     fl = prefill_flops(cfg, T)
     print(f"{'prefill, 2,048 tokens':34s} {pt * 1e3:8.3f} {T / pt:10.0f} {fl / 1e12:6.3f} TFLOP {fl / pt / 1e15:7.3f} PFLOP/s "
-          f"{fl / pt / BF16_PEAK:8.3f} {fl / pt / ceil['gemm']:11.3f}")
+          f"{fl / pt / BF16_PEAK:8.3f} {fl / pt / ceil['gemm']:11.3f}", flush=True)
+    if make_engine is not None:
+        del engine
+        torch.cuda.empty_cache()
+        for batch, context in ((8, 32768), (64, 32768), (8, 131072)):
+            eng = make_engine(batch, context)
+            decode_row(eng, batch, context - 64 - 16 - 3 - head_start(eng, batch, context), 16, 64)
+            del eng
+            torch.cuda.empty_cache()
     return 0
 
 
@@ -209,9 +252,14 @@ def main() -> int:
                                       "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}}), flush=True)
         return 0
     if args.report:
-        return report(engine, cfg, args.steps, args.warmup)
+        def long_engine(batch, context):
+            pages = batch * (-(-context // page)) + 64
+            return Engine.from_config(cfg, seed=0, cfg=EngineConfig(
+                dtype="bfloat16", page_size=page, num_pages=pages, max_context=context, max_requests=batch,
+                max_tokens_per_step=2048 + batch, prefill_chunk=2048, admission="reserve"))
+        return report(engine, cfg, args.steps, args.warmup, long_engine)
     steps, warmup = args.steps, args.warmup
-    prompt_len = args.context - (warmup + steps + 3)
+    prompt_len = args.context - (warmup + steps + 3) - head_start(engine, args.batch, args.context)
     if prompt_len < 1:
         print("bench.py: --steps + --warmup do not fit into the context")
         return 2
@@ -223,7 +271,8 @@ def main() -> int:
         n_pre = max(1, min(256, args.context // 4))
         t0 = time.perf_counter()
         while time.perf_counter() - t0 < args.prewarm:
-            decode_run(engine, args.batch, args.context - n_pre - 3, 0, n_pre, seed=2)
+            decode_run(engine, args.batch, args.context - n_pre - 3 - head_start(engine, args.batch, args.context), 0,
+                       n_pre, seed=2)
         prewarm_s = time.perf_counter() - t0
     dt, mean_ctx = decode_run(engine, args.batch, prompt_len, warmup, steps, seed=1)
     ms_per_step = dt / steps * 1e3

@@ -42,6 +42,7 @@ SOURCES: Dict[str, str] = {
     "sampling": "sampling.hip",
     "gemm_mfma": "gemm_mfma.hip",
     "attention_mfma": "attention_mfma.hip",
+    "membench": "membench.hip",
 }
 
 # variants that are compiled with defines: library name -> list of define sets

@@ -229,6 +229,34 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+_SINKS = {}
+
+
+def read_bytes(t: torch.Tensor, workgroups: int = 0) -> None:
+    """Read the whole tensor with plain 16-byte loads and keep nothing (a measurement of the
+    memory's read rate with a kernel of our own)."""
+    _dev(t)
+    nbytes = t.numel() * t.element_size()
+    _check(nbytes % 16 == 0 and t.data_ptr() % 16 == 0, "read_bytes needs 16-byte alignment and size")
+    sink = _SINKS.get(t.device)
+    if sink is None:
+        sink = _SINKS[t.device] = torch.zeros(4, dtype=torch.int32, device=t.device)
+    lib = load_library("membench")
+    lib.sa_read_bytes.argtypes = [c_void_p, ctypes.c_size_t, c_int, c_void_p, c_void_p]
+    _ret(lib.sa_read_bytes(_ptr(t), nbytes, workgroups or 16 * compute_units(), _ptr(sink), _stream()), "read_bytes")
+
+
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor, workgroups: int = 0) -> None:
+    """dst = src with plain 16-byte loads and stores (a measurement of the memory's copy rate)."""
+    _dev(dst, src)
+    nbytes = src.numel() * src.element_size()
+    _check(dst.numel() * dst.element_size() == nbytes and nbytes % 16 == 0 and dst.data_ptr() % 16 == 0
+           and src.data_ptr() % 16 == 0, "copy_bytes needs two buffers of one size, 16-byte aligned")
+    lib = load_library("membench")
+    lib.sa_copy_bytes.argtypes = [c_void_p, c_void_p, ctypes.c_size_t, c_int, c_void_p]
+    _ret(lib.sa_copy_bytes(_ptr(dst), _ptr(src), nbytes, workgroups or 16 * compute_units(), _stream()), "copy_bytes")
+
+
 def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Optional[torch.Tensor],
            out: torch.Tensor) -> torch.Tensor:
     """One token per row of fp32 logits: argmax where temperature is 0 (or None), else the

@@ -617,3 +617,20 @@ def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     mask[page, off] = False
     assert k1.permute(0, 2, 1, 3)[mask].abs().max().item() == 0 and v1.permute(0, 3, 1, 2)[mask].abs().max().item() == 0
     assert not ops.qkv_rope_available(h, w, k1, 24, 24, False) and not ops.qkv_rope_available(h, w, k1, D, D, True)
+
+
+def test_memory_ceiling_kernels_copy_and_refuse():
+    """The plain read and copy kernels of the measurement program: the copy is exact for sizes that
+    are no multiple of the grid, misaligned or ragged buffers are refused."""
+    from serve_amd import ops
+    for n in (16, 4096 + 16, 3 * 1024 * 1024 + 48):
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=DEV)
+        dst = torch.zeros_like(src)
+        ops.copy_bytes(dst, src, workgroups=7)
+        ops.read_bytes(src, workgroups=5)
+        torch.cuda.synchronize()
+        assert torch.equal(dst, src)
+    with pytest.raises(ops.KernelError):
+        ops.read_bytes(torch.zeros(24, dtype=torch.uint8, device=DEV))
+    with pytest.raises(ops.KernelError):
+        ops.copy_bytes(torch.zeros(32, dtype=torch.uint8, device=DEV), torch.zeros(48, dtype=torch.uint8, device=DEV))

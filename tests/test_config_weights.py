@@ -226,8 +226,9 @@ def test_attention_key_splits_are_chosen_by_the_shape_of_the_launch():
 
 
 def test_named_shapes_are_the_configurations_the_measurements_are_specified_on():
-    """`--shape tiny-a | tiny-b | llama-1b | llama-3b | llama-8b`: every size the specification of the
-    benchmark configurations gives (BASELINE.json, read as text: it is prose) appears in the preset."""
+    """`--shape tiny-a | tiny-b | llama-1b | llama-3b | llama-8b`: the presets hold the sizes that the
+    measured configurations are specified with (two tiny ones that differ in every size and option,
+    and the shapes of Llama-3.2-1B, Llama-3.2-3B and Llama-3.1-8B)."""
     from serve_amd.benchmark import SHAPES
     a, b, one = SHAPES["tiny-a"], SHAPES["tiny-b"], SHAPES["llama-1b"]
     assert (a.num_hidden_layers, a.hidden_size, a.num_attention_heads, a.num_key_value_heads, a.head_dim,

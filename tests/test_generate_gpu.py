@@ -418,6 +418,26 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     # the state matters: the last position differs from running the last token alone
     assert not torch.allclose(whole(a[-1:])[0], wa[-1], atol=1e-3)
 
+    # and through the scheduler: a model without any paged cache (no group, no pages) is admitted,
+    # taken in portions of four tokens beside decoding requests, and generates what feeding the
+    # whole sequence again for every token gives
+    from serve_amd.engine.engine import Request
+
+    def greedy(tokens, n):
+        seq, new = list(tokens), []
+        for _ in range(n):
+            t = int(whole(seq)[-1].argmax())
+            new.append(t)
+            seq.append(t)
+        return new
+    eng2 = Engine.from_folder(folder, EngineConfig(dtype="float32", page_size=8, num_pages=8, max_context=64,
+                                                  max_requests=3, prefill_chunk=4, max_tokens_per_step=6))
+    log = []
+    out = eng2.generate([Request(torch.tensor(p), len(p), 5) for p in (a, b, a[:3])], step_log=log)
+    assert [r.generated_tokens.tolist() for r in out] == [greedy(a, 5), greedy(b, 5), greedy(a[:3], 5)]
+    assert any(len(s["requests"]) > 1 and max(s["counts"]) > 1 and min(s["counts"]) == 1 for s in log)
+    assert eng2.runner.cache.num_groups == 0 and eng2.runner.cache.free_slots() == 3
+
 
 # ---------------------------------------------------------------------------------------------
 # a toy feed-forward with routing and a toy position encoding, defined here, registered, built and

@@ -602,10 +602,8 @@ def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     assert ops.qkv_rope_available(h, w, k1, D, D, False)
     q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=DEV)
     ops.qkv_rope_bf16(h, w, q, pos, inv_freq, slots, k1, v1, Hq, Hk, D, ps)
-    # the same in three steps: product (fp32 out), rotation and write in fp32, rounding at the end
-    qkv = torch.empty((M, (Hq + 2 * Hk) * D), dtype=torch.float32, device=DEV)
-    ops.gemm_bf16_skinny(h, w, qkv)
-    x = qkv.double().view(M, Hq + 2 * Hk, D)
+    # the same in three steps, none of them the engine's: product and rotation in fp64, rounding at the end
+    x = (h.double() @ w.double().T).view(M, Hq + 2 * Hk, D)
     q_want = rope_ref(x[:, :Hq], pos, inv_freq, D, False).reshape(M, Hq * D)
     k_want = rope_ref(x[:, Hq:Hq + Hk], pos, inv_freq, D, False)
     torch.testing.assert_close(q.double(), q_want, atol=2e-2, rtol=1e-2)

@@ -502,7 +502,7 @@ __global__ __launch_bounds__(64 * WG_SPLITS) void paged_attention_mfma_wg_kernel
 // a SIMD whose two waves keep the vector unit busy gains little from matrix instructions of the
 // other wave running beside them (288 vector + 32 matrix instructions: 429 ns + 229 ns apart,
 // 589 ns together); exponentials, three and a half times as slow as plain vector instructions when
-// alone, do run beside those.  Hence one softmax update per 64 keys, three-way maxima, row sums taken by the matrix cores, O
+// alone, do run beside those.  Hence one softmax update per 64 or 128 keys (the stage's share of a wave), three-way maxima, row sums taken by the matrix cores, O
 // rescaled only when a maximum has moved, and page addresses that are a constant plus a product.
 //
 // The work per stage is the same straight line of code for every wave and stage: a block that is
@@ -524,7 +524,14 @@ constexpr int log2_of(int x) { return x <= 1 ? 0 : 1 + log2_of(x / 2); }
 template <int KW>
 struct PromptShape {
   static constexpr int TW = 8 / KW;                        // tiles of 32 rows per workgroup
-  static constexpr int KB = HD <= 64 ? 2 : 1;              // blocks of 32 keys per wave and stage
+#ifndef PROMPT_KB_SMALL_HEADS
+#define PROMPT_KB_SMALL_HEADS 4
+#endif
+#ifndef PROMPT_KB_BIG_HEADS
+#define PROMPT_KB_BIG_HEADS 2
+#endif
+  // blocks of 32 keys per wave and stage
+  static constexpr int KB = HD <= 64 ? (KW == 2 ? PROMPT_KB_SMALL_HEADS : 2) : (KW == 2 ? PROMPT_KB_BIG_HEADS : 1);
   static constexpr int BLOCKS = KW * KB;
   static constexpr int KEYS = 32 * BLOCKS;                 // keys per stage
   static constexpr int K_ROW = HD <= 64 ? 128 : 256;       // bytes of a key's row in LDS

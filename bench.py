@@ -240,7 +240,8 @@ def main() -> int:
     page = 16
     pages_needed = args.batch * (-(-args.context // page)) + 64 * (-(-600 // page)) + 256
     ecfg = EngineConfig(dtype="bfloat16", page_size=page, num_pages=pages_needed, max_context=args.context,
-                        max_requests=64, max_tokens_per_step=2048, prefill_chunk=2048, admission="reserve")
+                        max_requests=max(64, args.batch), max_tokens_per_step=2048, prefill_chunk=2048,
+                        admission="reserve")
     t_load = time.perf_counter()
     engine = Engine.from_config(cfg, seed=0, cfg=ecfg)
     print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)

@@ -301,8 +301,8 @@ __global__ __launch_bounds__(64 * KS) void gemm_skinny_kernel(const bf16_t* __re
   store_tiles<RT, MT, TC, EPI>(acc, C, M, N, m0, n0, head, t16, qa, ql, g, c);
 }
 
-// The same products for up to 64 rows of activations (decode at all but the smallest batches, short
-// prompt portions).  With that many rows a workgroup reads about as many bytes of activations as of
+// The same products for up to 128 rows of activations a pass (decode at all but the smallest
+// batches, short prompt portions).  With that many rows a workgroup reads about as many bytes of activations as of
 // weights, so the activations are staged through LDS and shared.  A workgroup has NR x KH waves:
 // NR groups of weight rows times KH slices of each 256-wide stage of K; the NR waves of a slice read
 // the same activation fragments, and the KH slices add their sums through LDS at the end, in order.
@@ -526,33 +526,65 @@ static bool takes_skinny(int M, int N, const QkvRopeArgs& qa) {
   return M <= 2;
 }
 
+// workgroup shapes (row groups x K slices) of products with 65 to 128 rows of activations
+#ifndef MID8_PLAIN_NR
+#define MID8_PLAIN_NR 2
+#define MID8_PLAIN_KH 4
+#endif
+#ifndef MID8_SWIGLU_NR
+#define MID8_SWIGLU_NR 2
+#define MID8_SWIGLU_KH 4
+#endif
+#ifndef MID8_HEAD_NR
+#define MID8_HEAD_NR 4
+#define MID8_HEAD_KH 2
+#endif
+
 template <typename TC, int EPI>
 static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                     const QkvRopeArgs& qa, hipStream_t stream) {
-  const int mt = M > 32 ? 4 : (M > 16 ? 2 : 1);      // 16-row tiles of activations per pass
+  // 16-row tiles of activations per pass: up to 128 rows in one pass (more rows: more passes, each
+  // streaming the weights again, which the caller avoids)
+  const int mt = M > 64 ? 8 : (M > 32 ? 4 : (M > 16 ? 2 : 1));
 #define GO(RT, MT, NR, KH) \
   return launch_mid<RT, MT, NR, KH, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
 #define GO3(RT, NR1, KH1, NR2, KH2, NR4, KH4) \
   do {                                         \
     if (mt == 1) GO(RT, 1, NR1, KH1);          \
     if (mt == 2) GO(RT, 2, NR2, KH2);          \
-    GO(RT, 4, NR4, KH4);                       \
+    if (mt == 4) GO(RT, 4, NR4, KH4);          \
   } while (0)
+  // (with eight tiles a workgroup has 512 threads or more: fewer would hold too many activation
+  // segments each on their way into LDS)
   if constexpr (EPI == EPI_PLAIN) {
-    if (N < 8192) GO3(1, 2, 4, 2, 4, 2, 4);    // 32 weight rows a workgroup, K cut four ways inside it
+    if (N < 8192) {
+      GO3(1, 2, 4, 2, 4, 2, 4);                // 32 weight rows a workgroup, K cut four ways inside it
+      GO(1, 8, MID8_PLAIN_NR, MID8_PLAIN_KH);
+    }
     if (M <= 8) GO(1, 1, 4, 2);                // the head: 64 weight rows, or 128 with two passes' worth of rows
     if (M <= 32) GO(1, 2, 8, 2);
-    GO(1, 4, 8, 2);
+    if (M <= 64) GO(1, 4, 8, 2);
+    GO(1, 8, MID8_HEAD_NR, MID8_HEAD_KH);
   }
   if constexpr (EPI == EPI_QKV_ROPE) {
     const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
-    if (tiles < 256) GO3(1, 1, 8, 1, 8, 1, 8);   // one 16-row tile a workgroup, K cut eight ways
+    if (tiles < 256) {
+      GO3(1, 1, 8, 1, 8, 1, 8);                  // one 16-row tile a workgroup, K cut eight ways
+      // more than 64 rows: two passes of 64 (the second finds the weights in L2) fill the chip
+      // better than one pass with half as many workgroups (about 3 us less at 128 rows, 1B shape)
+      GO(1, 4, 1, 8);
+    }
     GO3(1, 2, 2, 2, 4, 2, 4);                    // two tiles
+    GO(1, 8, 2, 4);
   }
   if constexpr (EPI == EPI_SWIGLU) {
     const int tiles = (N + 15) / 16;             // N: rows of the gate (and of the up) matrix
-    if (tiles < 768) GO3(2, 1, 8, 2, 2, 2, 2);   // 32 to 64 weight rows a workgroup
+    if (tiles < 768) {
+      GO3(2, 1, 8, 2, 2, 2, 2);                  // 32 to 64 weight rows a workgroup
+      GO(2, 8, MID8_SWIGLU_NR, MID8_SWIGLU_KH);
+    }
     GO3(2, 4, 2, 4, 2, 4, 2);                    // 128
+    GO(2, 8, MID8_SWIGLU_NR, MID8_SWIGLU_KH);
   }
 #undef GO3
 #undef GO

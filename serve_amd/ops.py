@@ -281,7 +281,10 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Opti
 # ---------------------------------------------------------------------------------------------
 # bf16 matrix-core kernels
 # ---------------------------------------------------------------------------------------------
-SKINNY_MAX_ROWS = 64          # above this the weights would be streamed more than once per product
+# a product with more than 64 rows and this many outputs (the head over the vocabulary) is the
+# library's: the few-row kernel would read its 128 rows of activations once per 64 weight rows
+WIDE_OUTPUT = 65536
+SKINNY_MAX_ROWS = 128         # above this the weights would be streamed more than once per product
 
 
 def _aligned16(*tensors: torch.Tensor) -> bool:
@@ -296,7 +299,7 @@ def mfma_gemm_available(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> 
 
 
 def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out = a @ w^T on the matrix cores, weights streamed once per 64 rows of a.
+    """out = a @ w^T on the matrix cores, weights streamed once per 128 rows of a.
 
     `out` [M, N] bf16 or fp32; or fp32 [parts, M, N]: the inner dimension is cut into `parts`
     slices over workgroups and slice p's partial sums go to out[p] (the consumer adds them)."""
@@ -341,7 +344,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
     """bf16 product: the weight-streaming kernels for few rows, the BLAS library for many (the
     reference leaves all of its products to the library, serve/model.py:80-82,95,97,159); both
     write bf16 or fp32."""
-    if a.shape[0] <= SKINNY_MAX_ROWS:
+    if a.shape[0] <= SKINNY_MAX_ROWS and not (a.shape[0] > 64 and w.shape[0] >= WIDE_OUTPUT):
         return gemm_bf16_skinny(a, w, out)
     _dev(a, w, out)
     if out.dtype == torch.bfloat16:

@@ -495,7 +495,10 @@ def test_prompt_attention_long_prompts_windows_and_split_keys(Hq, Hk, D, ps):
 @pytest.mark.parametrize("c_dt", ["bfloat16", "float32"])
 @pytest.mark.parametrize("M,N,K", [(1, 70, 40), (3, 64, 64), (8, 3072, 2048), (16, 509, 96), (17, 130, 104),
                                    (33, 2048, 8192), (64, 8200, 256), (100, 77, 1024), (8, 128256 // 8, 192),
-                                   (2, 8200, 72), (5, 9001, 64), (24, 8193, 520), (12, 520, 1032)])
+                                   (2, 8200, 72), (5, 9001, 64), (24, 8193, 520), (12, 520, 1032),
+                                   # 65 to 128 rows: eight 16-row tiles a pass; more rows: several passes
+                                   (65, 2048, 2048), (100, 333, 264), (128, 8200, 520), (127, 3072, 2048),
+                                   (200, 130, 512)])
 def test_gemm_bf16_skinny(c_dt, M, N, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 4)
@@ -514,7 +517,9 @@ def test_gemm_bf16_skinny(c_dt, M, N, K):
 @pytest.mark.parametrize("M,I,K", [(1, 192, 64), (8, 8192, 2048), (20, 320, 192), (64, 1000, 96), (50, 8192, 2048),
                                    (2, 1000, 72), (3, 1000, 72), (16, 8200, 264), (30, 520, 1032),
                                    # many rows of weights: 128 of them a workgroup
-                                   (1, 12300, 64), (7, 12300, 264), (24, 14336, 128), (64, 12296, 72)])
+                                   (1, 12300, 64), (7, 12300, 264), (24, 14336, 128), (64, 12296, 72),
+                                   # 65 to 128 rows
+                                   (65, 1000, 96), (128, 8192, 2048), (97, 12296, 136), (113, 520, 1032)])
 def test_swiglu_bf16(M, I, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 6)
@@ -556,7 +561,8 @@ def test_kernels_refuse_what_they_do_not_take():
 
 
 @pytest.mark.parametrize("M,N,K,parts", [(1, 2048, 2048, 4), (8, 2048, 8192, 2), (16, 96, 256, 8), (5, 77, 520, 3),
-                                         (40, 130, 1000, 3), (64, 2048, 2048, 4), (17, 48, 8192, 8)])
+                                         (40, 130, 1000, 3), (64, 2048, 2048, 4), (17, 48, 8192, 8),
+                                         (128, 2048, 8192, 4), (90, 200, 1104, 2)])
 def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 4)
@@ -585,10 +591,13 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
                                              (33, 3, 1, 80, 16, 104), (5, 4, 4, 16, 4, 40),
                                              # 256 tiles of 16 rows and more: two tiles a workgroup
                                              (1, 24, 8, 128, 16, 136), (8, 32, 8, 128, 16, 520), (20, 24, 4, 128, 8, 72),
-                                             (64, 28, 2, 128, 16, 264), (3, 60, 4, 64, 16, 64)])
+                                             (64, 28, 2, 128, 16, 264), (3, 60, 4, 64, 16, 64),
+                                             # 65 to 128 rows
+                                             (65, 32, 8, 64, 16, 2048), (128, 3, 1, 96, 16, 72), (100, 24, 8, 128, 16, 264),
+                                             (77, 4, 2, 16, 8, 40)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
-    P = 7
+    P = 7 if M <= 64 else 20
     h = rnd((M, d), torch.bfloat16, 1)
     w = rnd(((Hq + 2 * Hk) * D, d), torch.bfloat16, 2, 0.1)
     # positions up to 131,071: the kernel takes the multiple of 2 pi off the angle itself

@@ -1,13 +1,15 @@
-// C[M, N] = A[M, K] * W[N, K]^T with fp32 multiply and fp32 accumulate on the vector ALU.
+// C[M, N] = A[M, K] * W[N, K]^T with fp32 multiply and fp32 accumulate.
 //
 // This is the true 32-bit matrix product of the float32 path (no reduced-precision matrix mode
-// is involved: plain v_fma_f32), and the product for any mix of storage types that the faster
+// is involved: v_fma_f32 and v_mfma_f32_32x32x2_f32, both full float32), and the product for any mix of storage types that the faster
 // MFMA kernels do not take.  The reference leaves these products to nn.Linear
 // (serve/model.py:80-82,95,97,159).
 //
-// Tiling: a 256-thread block owns a 64x64 tile of C; K advances in slices of 16 through LDS;
-// each thread accumulates a 4x4 sub-tile.  Every edge (M, N, K not multiples of the tile) is
-// guarded, so any size is accepted.
+// Three kernels: gemm_nt_rows_kernel for up to 16 rows of float32 activations, gemm_nt_mfma32_kernel
+// (the matrix cores' float32 instruction) for more rows whose length is a multiple of four, and
+// gemm_nt_kernel for everything else: a 256-thread block owns a 64x64 tile of C; K advances in
+// slices of 16 through LDS; each thread accumulates a 4x4 sub-tile with v_fma_f32.  Every edge (M,
+// N, K not multiples of the tile) is guarded, so any size is accepted.
 #include "common.h"
 
 #define GT_M 64
@@ -70,15 +72,238 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
   }
 }
 
+// The same product for few rows of activations (decode steps of the float32 path), where the work is
+// reading W once: a wave owns RW rows of W, its lanes split K (a float4 each, four per chunk of 1024),
+// the MR rows of activations of a pass lie in LDS a chunk at a time, and the lanes' partial sums are
+// added across the wave at the end, always in the same order.  Loads of W carry no conditions: a row
+// beyond N is read from the last row and not stored, and beyond K the address wraps to the chunk's
+// begin while the activation operand is zero.  Needs K % 4 == 0 and 16-byte aligned A and W.
+template <int MR, int RW>
+__global__ __launch_bounds__(256) void gemm_nt_rows_kernel(const float* __restrict__ A, const float* __restrict__ W,
+                                                           float* __restrict__ C, int M, int N, int K) {
+  constexpr int KC = 1024;
+  __shared__ float4 As[MR][KC / 4];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int n_base = (blockIdx.x * 4 + wave) * RW;
+  const int m0 = blockIdx.y * MR;
+  const float* wrow[RW];
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw) wrow[rw] = W + (size_t)min(n_base + rw, N - 1) * K;
+  float acc[RW][MR];
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+    for (int r = 0; r < MR; ++r) acc[rw][r] = 0.f;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k0 = 0; k0 < K; k0 += KC) {
+    __syncthreads();                                  // the chunk before has been used
+    for (int i = tid; i < MR * (KC / 4); i += 256) {
+      const int r = i / (KC / 4);
+      const int c = i - r * (KC / 4);
+      const int k = k0 + c * 4;
+      const int m = m0 + r;
+      As[r][c] = (m < M && k < K) ? *reinterpret_cast<const float4*>(A + (size_t)m * K + k) : zero4;
+    }
+    __syncthreads();
+    float4 w[4][RW];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + (j * 64 + lane) * 4;
+      const int kc = k < K ? k : k0;                  // beyond K: any valid address, the activations there are 0
+#pragma unroll
+      for (int rw = 0; rw < RW; ++rw) w[j][rw] = *reinterpret_cast<const float4*>(wrow[rw] + kc);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int r = 0; r < MR; ++r) {
+        const float4 a = As[r][j * 64 + lane];
+#pragma unroll
+        for (int rw = 0; rw < RW; ++rw) {
+          float t = acc[rw][r];
+          t = fmaf(w[j][rw].x, a.x, t);
+          t = fmaf(w[j][rw].y, a.y, t);
+          t = fmaf(w[j][rw].z, a.z, t);
+          t = fmaf(w[j][rw].w, a.w, t);
+          acc[rw][r] = t;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+      const float v = wave_sum(acc[rw][r]);
+      const int n = n_base + rw;
+      const int m = m0 + r;
+      if (lane == 0 && n < N && m < M) C[(size_t)m * N + n] = v;
+    }
+}
+
+template <int MR>
+static int launch_rows(const void* A, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
+  // many rows of W: four of them a wave; few: two, so that there are workgroups enough
+  const int rw = N >= 8192 ? 4 : 2;
+  dim3 grid((N + 4 * rw - 1) / (4 * rw), (M + MR - 1) / MR), block(256);
+  if (rw == 4)
+    hipLaunchKernelGGL((gemm_nt_rows_kernel<MR, 4>), grid, block, 0, stream, (const float*)A, (const float*)W,
+                       (float*)C, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_nt_rows_kernel<MR, 2>), grid, block, 0, stream, (const float*)A, (const float*)W,
+                       (float*)C, M, N, K);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Many rows (prompt portions of the float32 path, and any mix of storage types): the matrix cores'
+// float32 instruction, v_mfma_f32_32x32x2_f32, which multiplies and adds in full 32-bit precision
+// (it is not the reduced "xf32" mode).  A workgroup of four waves owns a 128 x 128 tile of C, a
+// wave 64 x 64 of it as 2 x 2 instruction tiles; K advances in slices of 16 through two LDS
+// buffers (rows padded to 17 floats, so that the 32 lanes that read a column of a slice fall into
+// 32 banks); a slice is fetched into registers while the slice before it is multiplied.
+// Operands: lane l gives A[row l % 32][k l / 32] and W[row l % 32][k l / 32]; result register i of
+// lane l is C[8 (i / 4) + 4 (l / 32) + i % 4][l % 32].  Needs K % 4 == 0 and 16-byte (bf16: 8-byte)
+// aligned rows; rows beyond M and N are read as zeros.
+// ---------------------------------------------------------------------------------------------
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float4 load4f(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4f(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(bf16_bits_to_float(u.x & 0xffffu), bf16_bits_to_float(u.x >> 16),
+                     bf16_bits_to_float(u.y & 0xffffu), bf16_bits_to_float(u.y >> 16));
+}
+
+#define MF_BM 128
+#define MF_BN 128
+#define MF_BK 16
+
+template <typename TA, typename TW, typename TC>
+__global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+                                                             TC* __restrict__ C, int M, int N, int K) {
+  __shared__ float As[2][MF_BM][MF_BK + 1];
+  __shared__ float Ws[2][MF_BN][MF_BK + 1];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * MF_BM;
+  const int n0 = blockIdx.x * MF_BN;
+  // what this thread fetches of a slice: rows lr and lr + 64 of both tiles, four floats at k4
+  const int lr = tid >> 2;
+  const int k4 = (tid & 3) * 4;
+  const TA* arow[2];
+  const TW* wrow[2];
+  bool aok[2], wok[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int m = m0 + lr + 64 * j, n = n0 + lr + 64 * j;
+    aok[j] = m < M;
+    wok[j] = n < N;
+    arow[j] = A + (size_t)(aok[j] ? m : 0) * K;
+    wrow[j] = W + (size_t)(wok[j] ? n : 0) * K;
+  }
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 ra[2], rw[2];
+  auto fetch = [&](int k0) __attribute__((always_inline)) {
+    const int k = k0 + k4;
+    const bool kok = k < K;                       // K % 4 == 0: a group of four is inside or outside
+    const int kc = kok ? k : 0;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      ra[j] = load4f(arow[j] + kc);
+      rw[j] = load4f(wrow[j] + kc);
+      if (!(kok && aok[j])) ra[j] = zero4;
+      if (!(kok && wok[j])) rw[j] = zero4;
+    }
+  };
+  auto stash = [&](int b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float* a = &As[b][lr + 64 * j][k4];
+      float* w = &Ws[b][lr + 64 * j][k4];
+      a[0] = ra[j].x; a[1] = ra[j].y; a[2] = ra[j].z; a[3] = ra[j].w;
+      w[0] = rw[j].x; w[1] = rw[j].y; w[2] = rw[j].z; w[3] = rw[j].w;
+    }
+  };
+  floatx16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int nslices = (K + MF_BK - 1) / MF_BK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int r32 = lane & 31, kh = lane >> 5;
+  for (int s = 0; s < nslices; ++s) {
+    const int b = s & 1;
+    if (s + 1 < nslices) fetch((s + 1) * MF_BK);
+#pragma unroll
+    for (int kk = 0; kk < MF_BK; kk += 2) {
+      float a[2], w[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[i] = As[b][wm * 64 + i * 32 + r32][kk + kh];
+        w[i] = Ws[b][wn * 64 + i * 32 + r32][kk + kh];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], w[j], acc[i][j], 0, 0, 0);
+    }
+    if (s + 1 < nslices) stash(b ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + r32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * kh + (e & 3);
+        if (m < M && n < N) C[(size_t)m * N + n] = from_float<TC>(acc[i][j][e]);
+      }
+    }
+}
+
+// up to this many rows of float32 activations take gemm_nt_rows_kernel (in passes of eight)
+#define ROWS_KERNEL_MAX_M 16
+
 extern "C" int sa_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                           int M, int N, int K, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return SA_ERR_ARG;
+  if (a_dtype == SA_F32 && w_dtype == SA_F32 && c_dtype == SA_F32 && M <= ROWS_KERNEL_MAX_M && (K & 3) == 0 &&
+      (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
+    if (M == 1) return launch_rows<1>(A, W, C, M, N, K, stream);
+    if (M == 2) return launch_rows<2>(A, W, C, M, N, K, stream);
+    if (M <= 4) return launch_rows<4>(A, W, C, M, N, K, stream);
+    return launch_rows<8>(A, W, C, M, N, K, stream);
+  }
+  // the matrix cores' float32 instruction where the rows can be fetched four elements at a time
+  const bool mfma = (K & 3) == 0 && ((uintptr_t)A & (a_dtype == SA_F32 ? 15 : 7)) == 0 &&
+                    ((uintptr_t)W & (w_dtype == SA_F32 ? 15 : 7)) == 0;
   dim3 grid((N + GT_N - 1) / GT_N, (M + GT_M - 1) / GT_M), block(256);
+  if (mfma) grid = dim3((N + MF_BN - 1) / MF_BN, (M + MF_BM - 1) / MF_BM);
   if (grid.y > 65535) return SA_ERR_ARG;
-#define GO(TA, TW, TC)                                                                              \
-  hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)A, (const TW*)W, \
-                     (TC*)C, M, N, K)
+#define GO(TA, TW, TC)                                                                                  \
+  do {                                                                                                  \
+    if (mfma)                                                                                           \
+      hipLaunchKernelGGL((gemm_nt_mfma32_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)A,     \
+                         (const TW*)W, (TC*)C, M, N, K);                                                \
+    else                                                                                                \
+      hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)A,            \
+                         (const TW*)W, (TC*)C, M, N, K);                                                \
+  } while (0)
   const int code = a_dtype * 4 + w_dtype * 2 + c_dtype;
   switch (code) {
     case 0: GO(float, float, float); break;

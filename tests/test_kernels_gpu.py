@@ -69,7 +69,12 @@ def test_add_rmsnorm(dtype, d, eps):
 
 @pytest.mark.parametrize("a_dt,w_dt,c_dt", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
                                             ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
-@pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 64, 64), (17, 130, 100), (64, 509, 96), (130, 65, 257)])
+@pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 64, 64), (17, 130, 100), (64, 509, 96), (130, 65, 257),
+                                   # up to 16 rows of float32 with K % 4 == 0: the weight-streaming kernel
+                                   (1, 2049, 2048), (8, 509, 1100), (16, 130, 8192), (5, 8200, 36), (2, 3, 4),
+                                   (9, 8193, 1028),
+                                   # more rows with K % 4 == 0: the matrix cores' float32 instruction
+                                   (200, 300, 2048), (129, 257, 64), (1000, 128, 512), (33, 40, 4), (128, 128, 16)])
 def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
     from serve_amd import ops
     a = rnd((M, K), DT[a_dt], 4)
@@ -77,7 +82,9 @@ def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
     out = torch.empty((M, N), dtype=DT[c_dt], device=DEV)
     ops.gemm_nt(a, w, out)
     want = a.double() @ w.double().T
-    torch.testing.assert_close(out.double(), want, **(tol("float32") if c_dt == "float32" else tol("bfloat16")))
+    # fp32 accumulation of K products of size ~0.1: the error grows with the square root of K
+    t32 = tol("float32") if K <= 257 else dict(atol=2e-6 * K ** 0.5, rtol=1e-5)
+    torch.testing.assert_close(out.double(), want, **(t32 if c_dt == "float32" else tol("bfloat16")))
 
 
 # ---------------------------------------------------------------------------------------------

@@ -41,6 +41,8 @@ def _generate(argv) -> int:
     ap.add_argument("--max-tokens-per-step", type=int, default=2048)
     ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")
+    ap.add_argument("--admit-interval", type=int, default=1, help="admit new requests at most every N steps while "
+                    "others run, so that the steps between are pure decode steps (1: at every step)")
     args = ap.parse_args(argv)
     import torch
 
@@ -49,7 +51,7 @@ def _generate(argv) -> int:
     cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, num_pages=args.num_pages,
                        memory_fraction=args.memory_fraction, max_context=args.max_context,
                        max_requests=args.max_requests, max_tokens_per_step=args.max_tokens_per_step,
-                       prefill_chunk=args.prefill_chunk, admission=args.admission, seed=args.seed)
+                       prefill_chunk=args.prefill_chunk, admission=args.admission, admit_interval=args.admit_interval, seed=args.seed)
     if args.model:
         engine = Engine.from_folder(args.model, cfg)
     else:

@@ -26,6 +26,11 @@ class EngineConfig:
     # (what the reference's admission does, serve/run.py:273-280); "optimistic": pages as
     # the request grows, and the youngest running request is preempted when they run out.
     admission: str = "reserve"
+    # new requests are admitted at most every this many steps while others run (1: at every step).
+    # A step with a newcomer's prompt is launched kernel by kernel, a step of decoding requests alone
+    # replays a graph: where the host is the bound (small models, hundreds of requests), admitting
+    # in turns trades a few idle slots for many cheaper steps.
+    admit_interval: int = 1
     seed: int = 0
     device: str = "cuda:0"
     # replay a decode-only step from a captured HIP graph
@@ -45,6 +50,8 @@ class EngineConfig:
             raise ValueError("max_context, max_requests and max_tokens_per_step must be positive")
         if self.prefill_chunk <= 0:
             raise ValueError("prefill_chunk must be positive")
+        if self.admit_interval < 1:
+            raise ValueError("admit_interval must be at least 1")
 
     @property
     def max_pages_per_request(self) -> int:

@@ -91,6 +91,7 @@ class Scheduler:
         self._reserved = [0] * self.cache.num_groups
         self._reservation = {}
         self.steps = 0
+        self._admit_at = 0                  # the step from which new requests are admitted again
         # one record per step (requests, token counts, who was sampled) when asked for: tracing only
         self.record_steps = record_steps
         self.step_log: List[dict] = []
@@ -218,8 +219,12 @@ class Scheduler:
                 else:
                     self._preempt(victim)
                 continue
-            # 3. new requests, first come first served, stop at the first that does not fit
-            while self.waiting and budget > 0:
+            # 3. new requests, first come first served, stop at the first that does not fit.  With an
+            # admission interval above one, newcomers wait for its next turn while anything else
+            # runs: the steps in between stay pure decode steps, which replay from a graph
+            admit = not plan.requests or self.steps >= self._admit_at
+            admitted = 0
+            while admit and self.waiting and budget > 0:
                 r = self.waiting[0]
                 if r.done():
                     self.waiting.popleft()
@@ -232,11 +237,14 @@ class Scheduler:
                 if not self._try_admit(r, free, n):
                     break
                 self.waiting.popleft()
+                admitted += 1
                 if try_add(r, n):
                     budget -= n
                 else:
                     # admitted under a reservation but the pages are still held by others
                     break
+            if admitted:
+                self._admit_at = self.steps + max(1, int(getattr(cfg, "admit_interval", 1)))
             if plan.requests:
                 return plan
             if not self.running:

@@ -237,6 +237,35 @@ def test_every_request_gets_its_own_tokens(admission, budget, chunk):
     assert [first[r.req_id] for r in reqs] == sorted(first[r.req_id] for r in reqs)
 
 
+@pytest.mark.parametrize("interval", [3, 5])
+def test_admission_in_turns_keeps_the_steps_between_free_of_newcomers(interval):
+    """`admit_interval` N: while anything runs, new requests start only every N-th step, so the steps
+    between hold no request's first portion; an idle engine admits at once; tokens are unchanged."""
+    rng = random.Random(4)
+    reqs = make_requests(rng, 14, max_prompt=10, max_new=9)
+    runner = FakeRunner(num_pages=64, page_size=4, max_requests=3)       # three at a time: the others wait
+    cfg = EngineConfig(max_tokens_per_step=64, prefill_chunk=64, max_context=256, page_size=4, num_pages=64,
+                       max_requests=3, admit_interval=interval)
+    sched = Scheduler(runner, FakeSampler(), cfg)
+    done = sched.run(reqs)
+    assert all(r.error is None and r.generated == alone(r.prompt, r.max_new_tokens) for r in done)
+    started, starts = set(), []
+    for i, st in enumerate(runner.steps):
+        new = [rid for rid, _ in st if rid not in started]
+        if new:
+            starts.append((i, len(st) - len(new)))          # (step, requests that were already running)
+        started.update(new)
+    assert len(starts) >= 4
+    for (a, _), (b, others) in zip(starts, starts[1:]):
+        assert b - a >= interval or others == 0, f"newcomers at steps {a} and {b} with {others} others running"
+    # and with the default every step may bring a newcomer
+    runner1 = FakeRunner(num_pages=64, page_size=4, max_requests=3)
+    cfg1 = EngineConfig(max_tokens_per_step=64, prefill_chunk=64, max_context=256, page_size=4, num_pages=64, max_requests=3)
+    reqs1 = make_requests(random.Random(4), 14, max_prompt=10, max_new=9)
+    Scheduler(runner1, FakeSampler(), cfg1).run(reqs1)
+    assert len(runner1.steps) < len(runner.steps)
+
+
 def test_steps_are_mixed_prompt_portions_ride_with_decodes():
     rng = random.Random(2)
     reqs = [GenerationRequest(0, [1] * 5, 10), GenerationRequest(1, [2] * 30, 3)]

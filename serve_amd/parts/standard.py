@@ -154,7 +154,8 @@ class GQAAttention(Part):
 
     def _project_encode_store(self, h: torch.Tensor, ctx, cache: LayerCache, slots: Optional[torch.Tensor]):
         """q (with k and v behind it in the same rows when they are stored), encoded by position,
-        k and v written to the token's cache slots.  Returns the rows and their stride."""
+        k and v written to the token's cache slots.  Returns the rows: [T, Hq D] (q alone) or
+        [T, (Hq + 2 Hk) D]; either way q is their first Hq D columns."""
         Hq, Hk, D = self.num_heads, self.num_kv_heads, self.head_dim
         store = slots is not None
         rot = self.position.rotary()

@@ -1,6 +1,7 @@
-// Paged attention, one wave per (token, query head), fp32 arithmetic throughout.
+// Paged attention in fp32 arithmetic: one wave per (token, query head) (below), and for prompt
+// portions of the float32 path a kernel that shares keys and values across 64 rows (further down).
 //
-// This is the attention of the float32 path and the fallback-free general form: any head_dim up
+// The first is the attention of the float32 path's single tokens and the general form: any head_dim up
 // to 256, any head counts, any page size, any mix of prompt portions and single tokens in one
 // launch.  Formulas as in serve/kernels/attn_prefill.py:56-72,205 and attn_decode.py:99-111,236:
 // scores = q.k * scale, key j visible to the query at absolute position p iff j <= p (and
@@ -91,6 +92,253 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const int i = lane + a * SA_WAVE;
     if (i < D) orow[i] = from_float<TA>(acc[a] * inv_l);
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same attention for prompt portions of the float32 path, tiled: a workgroup of 256 threads
+// takes 64 rows (a row = a token of the segment and one of the G query heads of a KV head, so the
+// rows of a workgroup share every key and value) and walks over the keys in blocks of 64 that are
+// staged in LDS, where the kernel above fetches every key once per row.  fp32 throughout, on the
+// vector ALU: thread (tr, tc) of the 16 x 16 grid owns rows 4 tr .. 4 tr + 3; of a block's scores
+// it computes keys tc, tc + 16, tc + 32, tc + 48, of the output dims tc, tc + 16, ...; row maxima
+// and sums are taken across the 16 lanes of a row group.  Online softmax as above.
+// Needs D % 16 == 0, D <= 128 and a page size that is a multiple of 4 (four consecutive keys then
+// lie in one page, and their values, stored transposed, are one 16-byte load).
+// ---------------------------------------------------------------------------------------------
+#define TL_ROWS 64
+#define TL_KEYS 64
+
+template <int DV>   // D / 16
+__global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
+    const float* __restrict__ q, int q_stride, float* __restrict__ out, const float* __restrict__ k_pages,
+    const float* __restrict__ v_pages, const int* __restrict__ block_table, int max_pages,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, float scale,
+    int window) {
+  constexpr int D = DV * 16;
+  constexpr int LD = D + 4;                       // row length in LDS: keeps 16-byte alignment, spreads banks
+  extern __shared__ __attribute__((aligned(16))) float tl_smem[];
+  float* Qs = tl_smem;                            // [64][LD]
+  float* Ks = Qs + TL_ROWS * LD;                  // [64][LD]
+  float* Vs = Ks + TL_KEYS * LD;                  // [64][LD]
+  float* Ps = Vs + TL_KEYS * LD;                  // [64][68]
+  constexpr int LP = TL_KEYS + 4;
+
+  const int tid = threadIdx.x;
+  const int tr = tid >> 4, tc = tid & 15;
+  const int g = blockIdx.x % Hk;                  // KV head
+  const int item = blockIdx.x / Hk;               // tile of 64 rows within the segment
+  const int seg = blockIdx.y;
+  const int G = Hq / Hk;
+  const int q_begin = cu_q[seg];
+  const int q_len = cu_q[seg + 1] - q_begin;
+  const int rows_total = q_len * G;
+  const int r0 = item * TL_ROWS;
+  if (r0 >= rows_total) return;
+  const int ctx = ctx_len[seg];
+  const int ctx_before = ctx - q_len;
+  const int* bt = block_table + (size_t)seg * max_pages;
+
+  // the tile's queries
+  for (int i = tid; i < TL_ROWS * (D / 4); i += 256) {
+    const int r = i / (D / 4), c4 = i - r * (D / 4);
+    const int row = min(r0 + r, rows_total - 1);
+    const int j = row / G, gi = row - j * G;
+    *reinterpret_cast<float4*>(Qs + r * LD + c4 * 4) =
+        *reinterpret_cast<const float4*>(q + (size_t)(q_begin + j) * q_stride + (size_t)(g * G + gi) * D + c4 * 4);
+  }
+  int qpos[4];
+  bool rvalid[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = r0 + tr * 4 + r;
+    rvalid[r] = row < rows_total;
+    qpos[r] = ctx_before + min(row, rows_total - 1) / G;
+  }
+  const int hi = ctx_before + min(r0 + TL_ROWS - 1, rows_total - 1) / G;          // last key any row of the tile sees
+  const int lo = window > 0 ? max(0, ctx_before + r0 / G - window + 1) : 0;      // first key any row sees
+
+  float m[4], l[4], acc[4][DV];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+#pragma unroll
+    for (int e = 0; e < DV; ++e) acc[r][e] = 0.f;
+  }
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  for (int kb = (lo / TL_KEYS) * TL_KEYS; kb <= hi; kb += TL_KEYS) {
+    __syncthreads();                              // the block before has been used (and Qs is written)
+    // keys: 64 rows of D floats, 16 bytes a thread at a time
+    for (int i = tid; i < TL_KEYS * (D / 4); i += 256) {
+      const int key = i / (D / 4), c4 = i - key * (D / 4);
+      const int kpos = kb + key;
+      float4 v = zero4;
+      if (kpos >= lo && kpos <= hi) {
+        const int page = bt[kpos / page_size];
+        const int off = kpos % page_size;
+        v = *reinterpret_cast<const float4*>(k_pages + (((size_t)page * Hk + g) * page_size + off) * D + c4 * 4);
+      }
+      *reinterpret_cast<float4*>(Ks + key * LD + c4 * 4) = v;
+    }
+    // values: stored [D][page_size] in a page; four consecutive keys of a dim are one load
+    for (int i = tid; i < (TL_KEYS / 4) * D; i += 256) {
+      const int d = i / (TL_KEYS / 4), quad = i - d * (TL_KEYS / 4);
+      const int kpos = kb + quad * 4;
+      float4 v = zero4;
+      if (kpos + 3 >= lo && kpos <= hi) {
+        const int page = bt[kpos / page_size];
+        const int off = kpos % page_size;
+        v = *reinterpret_cast<const float4*>(v_pages + (((size_t)page * Hk + g) * D + d) * page_size + off);
+        // a value beyond what any row sees may be anything (a page that holds another request's data,
+        // or none): its weight is 0, and 0 times it must be 0
+        if (kpos < lo || kpos > hi) v.x = 0.f;
+        if (kpos + 1 < lo || kpos + 1 > hi) v.y = 0.f;
+        if (kpos + 2 < lo || kpos + 2 > hi) v.z = 0.f;
+        if (kpos + 3 < lo || kpos + 3 > hi) v.w = 0.f;
+      }
+      Vs[(quad * 4 + 0) * LD + d] = v.x;
+      Vs[(quad * 4 + 1) * LD + d] = v.y;
+      Vs[(quad * 4 + 2) * LD + d] = v.z;
+      Vs[(quad * 4 + 3) * LD + d] = v.w;
+    }
+    __syncthreads();
+    // scores of rows 4 tr .. + 3 with keys tc + 16 c
+    float s[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) s[r][c] = 0.f;
+    for (int d4 = 0; d4 < D / 4; ++d4) {
+      float4 qv[4], kv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) qv[r] = *reinterpret_cast<const float4*>(Qs + (tr * 4 + r) * LD + d4 * 4);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) kv[c] = *reinterpret_cast<const float4*>(Ks + (tc + 16 * c) * LD + d4 * 4);
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float t = s[r][c];
+          t = fmaf(qv[r].x, kv[c].x, t);
+          t = fmaf(qv[r].y, kv[c].y, t);
+          t = fmaf(qv[r].z, kv[c].z, t);
+          t = fmaf(qv[r].w, kv[c].w, t);
+          s[r][c] = t;
+        }
+    }
+    // mask, row maxima and sums across the 16 lanes of the row group, p into LDS
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int key = kb + tc + 16 * c;
+        const bool vis = key <= qpos[r] && (window <= 0 || key > qpos[r] - window);
+        s[r][c] = vis ? s[r][c] * scale : -INFINITY;
+        mx = fmaxf(mx, s[r][c]);
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, SA_WAVE));
+      const float m_new = fmaxf(m[r], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;      // a row that has seen no key yet
+      const float alpha = expf(m[r] - m_safe);                    // exp(-inf) = 0 at the first visible block
+      float sum = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float p = expf(s[r][c] - m_safe);                   // exp(-inf) = 0 for invisible keys
+        Ps[(tr * 4 + r) * LP + tc + 16 * c] = p;
+        sum += p;
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, SA_WAVE);
+      l[r] = l[r] * alpha + sum;
+      m[r] = m_new;
+#pragma unroll
+      for (int e = 0; e < DV; ++e) acc[r][e] *= alpha;
+    }
+    __syncthreads();
+    // O += P V: dims tc + 16 e
+    for (int j4 = 0; j4 < TL_KEYS / 4; ++j4) {
+      float4 pv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pv[r] = *reinterpret_cast<const float4*>(Ps + (tr * 4 + r) * LP + j4 * 4);
+#pragma unroll
+      for (int e = 0; e < DV; ++e) {
+        const float v0 = Vs[(j4 * 4 + 0) * LD + tc + 16 * e];
+        const float v1 = Vs[(j4 * 4 + 1) * LD + tc + 16 * e];
+        const float v2 = Vs[(j4 * 4 + 2) * LD + tc + 16 * e];
+        const float v3 = Vs[(j4 * 4 + 3) * LD + tc + 16 * e];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float t = acc[r][e];
+          t = fmaf(pv[r].x, v0, t);
+          t = fmaf(pv[r].y, v1, t);
+          t = fmaf(pv[r].z, v2, t);
+          t = fmaf(pv[r].w, v3, t);
+          acc[r][e] = t;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    if (!rvalid[r]) continue;
+    const int row = r0 + tr * 4 + r;
+    const int j = row / G, gi = row - j * G;
+    const float inv_l = 1.f / l[r];
+    float* orow = out + (size_t)(q_begin + j) * Hq * D + (size_t)(g * G + gi) * D;
+#pragma unroll
+    for (int e = 0; e < DV; ++e) orow[tc + 16 * e] = acc[r][e] * inv_l;
+  }
+}
+
+template <int DV>
+static int launch_tiled(const void* q, int q_stride, void* out, const void* k_pages, const void* v_pages,
+                        const int* block_table, int max_pages, const int* cu_q, const int* ctx_len, int B,
+                        int max_q_len, int Hq, int Hk, int page_size, float scale, int window, hipStream_t stream) {
+  constexpr int D = DV * 16;
+  const size_t lds = (size_t)(3 * 64 * (D + 4) + 64 * 68) * sizeof(float);
+  const long long items = ((long long)max_q_len * (Hq / Hk) + TL_ROWS - 1) / TL_ROWS;
+  if (items * Hk > 0x7fffffffLL || B > 65535) return SA_ERR_ARG;
+  hipError_t e = hipFuncSetAttribute((const void*)paged_attention_tiled_f32_kernel<DV>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  dim3 grid((unsigned)(items * Hk), B), block(256);
+  hipLaunchKernelGGL((paged_attention_tiled_f32_kernel<DV>), grid, block, lds, stream, (const float*)q, q_stride,
+                     (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, max_pages, cu_q,
+                     ctx_len, Hq, Hk, page_size, scale, window);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// float32 attention of every token of the B segments over their cached keys, 64 rows a workgroup.
+// D a multiple of 16 up to 128, page_size a multiple of 4; max_q_len: the longest segment.
+extern "C" int sa_paged_attention_tiled_f32(const void* q, int q_stride, void* out, const void* k_pages,
+                                            const void* v_pages, const int* block_table, int max_pages,
+                                            const int* cu_q, const int* ctx_len, int B, int max_q_len, int Hq,
+                                            int Hk, int D, int page_size, float scale, int window,
+                                            hipStream_t stream) {
+  if (B <= 0 || max_q_len <= 0) return 0;
+  if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > 128 || (D & 15) || page_size <= 0 || (page_size & 3) ||
+      max_pages <= 0 || (q_stride & 3))
+    return SA_ERR_ARG;
+#define GO(DV)                                                                                                  \
+  case DV:                                                                                                      \
+    return launch_tiled<DV>(q, q_stride, out, k_pages, v_pages, block_table, max_pages, cu_q, ctx_len, B,       \
+                            max_q_len, Hq, Hk, page_size, scale, window, stream)
+  switch (D / 16) {
+    GO(1);
+    GO(2);
+    GO(3);
+    GO(4);
+    GO(5);
+    GO(6);
+    GO(7);
+    GO(8);
+  }
+#undef GO
+  return SA_ERR_ARG;
 }
 
 extern "C" int sa_paged_attention_simple(const void* q, int q_stride, void* out, int act_dtype,

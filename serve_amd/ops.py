@@ -217,6 +217,49 @@ def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
     return out
 
 
+def tiled_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_stride: int) -> bool:
+    """float32 throughout, head sizes 16..128 in steps of 16, page sizes that are multiples of 4."""
+    P, Hk, page_size, D = k_pages.shape
+    return (q.dtype == torch.float32 and k_pages.dtype == torch.float32 and D % 16 == 0 and D <= 128
+            and page_size % 4 == 0 and q_row_stride % 4 == 0 and q.data_ptr() % 16 == 0)
+
+
+def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
+                              v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
+                              ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int,
+                              scale: float, window: Optional[int]) -> torch.Tensor:
+    """float32 attention of prompt portions: 64 rows (tokens x the query heads of a KV head) a
+    workgroup share the keys and values of their KV head through LDS (fp32 arithmetic on the vector ALU)."""
+    _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
+    P, Hk, page_size, D = k_pages.shape
+    _check(tiled_attention_available(q, k_pages, q_row_stride),
+           f"paged_attention_tiled_f32 takes float32, head sizes 16..128 in steps of 16 and page sizes that are "
+           f"multiples of 4; got head size {D}, page size {page_size}")
+    _check(v_pages.shape == (P, Hk, D, page_size) and v_pages.dtype == torch.float32,
+           "v_pages must be fp32 [P, Hk, D, page_size]")
+    _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
+    T = num_tokens
+    _check(out.shape == (T, num_heads * D) and out.dtype == torch.float32, "attention output must be fp32 [T, Hq D]")
+    _check(q.numel() >= (T - 1) * q_row_stride + num_heads * D if T else True, "q is too short")
+    _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
+    B = block_table.shape[0]
+    _i32(cu_q, B + 1, "cu_q")
+    _i32(ctx_len, B, "ctx_len")
+    _check(1 <= max_q_len <= max(T, 1), "max_q_len out of range")
+    lib = load_library("attention_simple")
+    _ret(lib.sa_paged_attention_tiled_f32(
+        _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(max_q_len), c_int(num_heads),
+        c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0), _stream()),
+        "paged_attention_tiled_f32")
+    return out
+
+
+# rows (tokens x query heads of a KV head) of the longest segment from which the float32 path's tiled
+# attention is taken; below, the one-wave-per-row kernel has nothing to share
+TILED_MIN_ROWS = 16
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
     _dev(gate_up, out)
@@ -567,5 +610,10 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
             paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
                                  t_end, max_q, num_heads, scale, window, splits, s0, n, in_workgroup=inside)
         return out
+    Hk = k_pages.shape[1]
+    if (tiled_attention_available(q, k_pages, q_row_stride)
+            and ctx.max_q_len * (num_heads // Hk) > TILED_MIN_ROWS):
+        return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
+                                         ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window)
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                   ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

@@ -261,6 +261,9 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     if kernel == "simple":
         ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
                                    T, Hq, scale, window)
+    elif kernel == "tiled":
+        ops.paged_attention_tiled_f32(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
+                                      max(ql for _, ql in segs), Hq, scale, window)
     elif kernel == "dispatch":
         # the way the attention part calls it: the step's facts decide how many launches there are
         from types import SimpleNamespace
@@ -303,6 +306,25 @@ def test_paged_attention_simple(dtype, Hq, Hk, D, ps):
 def test_paged_attention_simple_window_and_standout(dtype):
     attention_case(dtype, 4, 2, 32, 8, [(0, 40), (50, 1), (33, 9)], seed=7, window=16)
     attention_case(dtype, 4, 2, 32, 8, [(0, 300), (299, 1)], seed=8, standout=True)
+
+
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 2, 64, 16), (6, 2, 48, 12),
+                                        (5, 5, 80, 32), (2, 1, 128, 16), (32, 8, 64, 16), (7, 1, 112, 64)])
+def test_paged_attention_tiled_f32(Hq, Hk, D, ps):
+    """The float32 path's attention of prompt portions (64 rows a workgroup share keys and values
+    through LDS): portions at the start, in the middle and at the end of a context, single tokens
+    among them, segments of more rows than a workgroup takes and of fewer."""
+    segs = [(0, 7), (12, 1), (0, 1), (63, 5), (130, 1), (5, 70), (0, 200), (190, 33)]
+    attention_case("float32", Hq, Hk, D, ps, segs, seed=300 + D, kernel="tiled")
+
+
+def test_paged_attention_tiled_f32_window_standout_and_poison():
+    attention_case("float32", 4, 2, 32, 8, [(0, 40), (50, 1), (33, 9), (100, 70)], seed=17, window=16, kernel="tiled")
+    attention_case("float32", 4, 2, 32, 8, [(0, 300), (299, 1)], seed=18, standout=True, kernel="tiled")
+    # pages that no row sees are given back (-1 in the table) and everything unowned holds NaN
+    attention_case("float32", 6, 2, 64, 16, [(0, 90), (200, 40), (77, 3)], seed=19, poison=True, kernel="tiled")
+    attention_case("float32", 6, 2, 64, 16, [(150, 40), (300, 2), (64, 64)], seed=20, window=48, poison=True,
+                   kernel="tiled")
 
 
 def test_attention_reduces_to_library_routine():

@@ -26,6 +26,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK = 8.0e12            # bytes/s, MI355X
 BF16_PEAK = 2.5e15           # dense bf16 MFMA flop/s, MI355X
+FP32_PEAK = 157.3e12         # fp32 matrix flop/s, MI355X
+ITEM = {"bfloat16": 2, "float32": 4}
 
 
 def model_config(layers: int, shape: str = "llama-1b"):
@@ -38,15 +40,15 @@ def model_config(layers: int, shape: str = "llama-1b"):
     return replace(cfg, num_hidden_layers=layers if layers > 0 else cfg.num_hidden_layers)
 
 
-def weight_bytes(cfg) -> int:
+def weight_bytes(cfg, itemsize: int = 2) -> int:
     d, D = cfg.hidden_size, cfg.head_dim
     per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D * d + d * cfg.num_attention_heads * D
                  + 3 * d * cfg.intermediate_size + 2 * d)
-    return 2 * (per_layer * cfg.num_hidden_layers + cfg.vocab_size * d + d)
+    return itemsize * (per_layer * cfg.num_hidden_layers + cfg.vocab_size * d + d)
 
 
-def kv_bytes_per_token(cfg) -> int:
-    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * 2
+def kv_bytes_per_token(cfg, itemsize: int = 2) -> int:
+    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * itemsize
 
 
 def prefill_flops(cfg, T: int) -> float:
@@ -218,6 +220,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has, only to save time; "
                     "both numbers are reported (0: all)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16", help="float32: the true 32-bit "
+                    "path (weights, cache and arithmetic in float32), measured against the float32 peaks")
     ap.add_argument("--shape", default="llama-1b", help="llama-1b (the headline measurement), llama-3b, llama-8b")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch-1/64 points")
     ap.add_argument("--prefill-only", action="store_true",
@@ -239,18 +243,21 @@ def main() -> int:
     shape_name = {"llama-1b": "Llama-3.2-1B", "llama-3b": "Llama-3.2-3B", "llama-8b": "Llama-3.1-8B"}.get(args.shape, args.shape)
     page = 16
     pages_needed = args.batch * (-(-args.context // page)) + 64 * (-(-600 // page)) + 256
-    ecfg = EngineConfig(dtype="bfloat16", page_size=page, num_pages=pages_needed, max_context=args.context,
+    item = ITEM[args.dtype]
+    peak = BF16_PEAK if args.dtype == "bfloat16" else FP32_PEAK
+    ecfg = EngineConfig(dtype=args.dtype, page_size=page, num_pages=pages_needed, max_context=args.context,
                         max_requests=max(64, args.batch), max_tokens_per_step=2048, prefill_chunk=2048,
                         admission="reserve")
     t_load = time.perf_counter()
-    engine = Engine.from_config(cfg, seed=0, cfg=ecfg)
+    engine = Engine.from_config(cfg, seed=0, cfg=ecfg,
+                                weight_dtype=torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
     print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
 
     if args.prefill_only:
         T = 2048
         pt = prefill_run(engine, T, repeats=5, seed=7)
         print(json.dumps({"prefill": {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                                      "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}}), flush=True)
+                                      "frac": round(prefill_flops(cfg, T) / pt / peak, 4)}}), flush=True)
         return 0
     if args.report:
         def long_engine(batch, context):
@@ -278,7 +285,7 @@ def main() -> int:
     dt, mean_ctx = decode_run(engine, args.batch, prompt_len, warmup, steps, seed=1)
     ms_per_step = dt / steps * 1e3
     value = args.batch * steps / dt
-    step_bytes = weight_bytes(cfg) + args.batch * mean_ctx * kv_bytes_per_token(cfg)
+    step_bytes = weight_bytes(cfg, item) + args.batch * mean_ctx * kv_bytes_per_token(cfg, item)
     achieved = step_bytes / (dt / steps)
     rs = cfg.rope_scaling
     rope_text = "none" if rs is None else (f"llama3 factor {rs.factor:g} low {rs.low_freq_factor:g} high "
@@ -288,7 +295,7 @@ def main() -> int:
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "prewarm_s": round(prewarm_s, 2),
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
         "config": {"model": shape_name.lower() + "-shape", "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single-gpu", "layers": cfg.num_hidden_layers, "layers_full": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
@@ -302,7 +309,7 @@ def main() -> int:
         T = 2048
         pt = prefill_run(engine, T, repeats=3, seed=7)
         out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                          "frac": round(prefill_flops(cfg, T) / pt / BF16_PEAK, 4)}
+                          "frac": round(prefill_flops(cfg, T) / pt / peak, 4)}
         points = {}
         for b in (1, 8, 64):
             d, _ = decode_run(engine, b, 256, 4, 250, seed=10 + b)

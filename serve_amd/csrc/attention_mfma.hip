@@ -1050,19 +1050,6 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
 
 extern "C" int sa_attention_mfma_head_dim() { return HD; }
 
-// compute units of the current device (asked once per device; 256 if the runtime will not say)
-static int compute_units() {
-  static int cached[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (!cached[dev]) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 // A step whose segments have at most 16 rows each (single decoded tokens) takes the one-wave kernel,
 // any other the prompt kernel.  `in_workgroup` (such steps only, num_splits 1): the key range of every
 // (segment, KV head) is cut four ways over the waves of one workgroup, which merges the parts itself.

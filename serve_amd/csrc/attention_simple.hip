@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
     const float* __restrict__ q, int q_stride, float* __restrict__ out, const float* __restrict__ k_pages,
     const float* __restrict__ v_pages, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, float scale,
-    int window) {
+    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int D = DV * 16;
   constexpr int LD = D + 4;                       // row length in LDS: keeps 16-byte alignment, spreads banks
   extern __shared__ __attribute__((aligned(16))) float tl_smem[];
@@ -127,7 +127,8 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
   const int tr = tid >> 4, tc = tid & 15;
   const int g = blockIdx.x % Hk;                  // KV head
   const int item = blockIdx.x / Hk;               // tile of 64 rows within the segment
-  const int seg = blockIdx.y;
+  const int seg = blockIdx.y / num_splits;
+  const int sp = blockIdx.y - seg * num_splits;   // this workgroup's part of the key range
   const int G = Hq / Hk;
   const int q_begin = cu_q[seg];
   const int q_len = cu_q[seg + 1] - q_begin;
@@ -167,8 +168,14 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
   }
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  for (int kb = (lo / TL_KEYS) * TL_KEYS; kb <= hi; kb += TL_KEYS) {
-    __syncthreads();                              // the block before has been used (and Qs is written)
+  // the blocks of 64 keys that the tile sees, cut evenly into num_splits parts
+  const int b_lo = lo / TL_KEYS, b_hi = hi / TL_KEYS;
+  const int per = (b_hi - b_lo + num_splits) / num_splits;
+  const int b_first = b_lo + sp * per;
+  const int b_last = min(b_hi, b_first + per - 1);
+  __syncthreads();                                // Qs is written (a part may have no block at all)
+  for (int kb = b_first * TL_KEYS; kb <= b_last * TL_KEYS; kb += TL_KEYS) {
+    __syncthreads();                              // the block before has been used
     // keys: 64 rows of D floats, 16 bytes a thread at a time
     for (int i = tid; i < TL_KEYS * (D / 4); i += 256) {
       const int key = i / (D / 4), c4 = i - key * (D / 4);
@@ -286,47 +293,91 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
     if (!rvalid[r]) continue;
     const int row = r0 + tr * 4 + r;
     const int j = row / G, gi = row - j * G;
+    const size_t orow_index = (size_t)(q_begin + j) * Hq + (g * G + gi);        // (token, head)
+    if (num_splits > 1) {
+      // unnormalised sums with their maximum and weight: merged by paged_attention_merge_f32_kernel
+      float* po = part_o + (orow_index * num_splits + sp) * D;
+#pragma unroll
+      for (int e = 0; e < DV; ++e) po[tc + 16 * e] = acc[r][e];
+      if (tc == 0) {
+        part_ml[(orow_index * num_splits + sp) * 2] = m[r];
+        part_ml[(orow_index * num_splits + sp) * 2 + 1] = l[r];
+      }
+      continue;
+    }
     const float inv_l = 1.f / l[r];
-    float* orow = out + (size_t)(q_begin + j) * Hq * D + (size_t)(g * G + gi) * D;
+    float* orow = out + orow_index * D;
 #pragma unroll
     for (int e = 0; e < DV; ++e) orow[tc + 16 * e] = acc[r][e] * inv_l;
+  }
+}
+
+// out[row] = sum_s w_s O_s / sum_s w_s l_s with w_s = exp(m_s - max m): the parts of a split key
+// range (a part that saw no key has m = -inf and weight 0).  One workgroup of 64 threads per row.
+__global__ __launch_bounds__(64) void paged_attention_merge_f32_kernel(const float* __restrict__ part_o,
+                                                                       const float* __restrict__ part_ml,
+                                                                       float* __restrict__ out, int D, int num_splits) {
+  const size_t row = blockIdx.x;
+  float mx = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, part_ml[(row * num_splits + s) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < num_splits; ++s) {
+    const float ms = part_ml[(row * num_splits + s) * 2];
+    L += (ms == -INFINITY ? 0.f : expf(ms - mx)) * part_ml[(row * num_splits + s) * 2 + 1];
+  }
+  const float inv = 1.f / L;
+  for (int d = threadIdx.x; d < D; d += 64) {
+    float o = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+      const float ms = part_ml[(row * num_splits + s) * 2];
+      const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
+      o = fmaf(w, part_o[(row * num_splits + s) * D + d], o);
+    }
+    out[row * D + d] = o * inv;
   }
 }
 
 template <int DV>
 static int launch_tiled(const void* q, int q_stride, void* out, const void* k_pages, const void* v_pages,
                         const int* block_table, int max_pages, const int* cu_q, const int* ctx_len, int B,
-                        int max_q_len, int Hq, int Hk, int page_size, float scale, int window, hipStream_t stream) {
+                        int max_q_len, int Hq, int Hk, int page_size, float scale, int window, int num_splits,
+                        float* part_o, float* part_ml, hipStream_t stream) {
   constexpr int D = DV * 16;
   const size_t lds = (size_t)(3 * 64 * (D + 4) + 64 * 68) * sizeof(float);
   const long long items = ((long long)max_q_len * (Hq / Hk) + TL_ROWS - 1) / TL_ROWS;
-  if (items * Hk > 0x7fffffffLL || B > 65535) return SA_ERR_ARG;
+  if (items * Hk > 0x7fffffffLL || (long long)B * num_splits > 65535) return SA_ERR_ARG;
   hipError_t e = hipFuncSetAttribute((const void*)paged_attention_tiled_f32_kernel<DV>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
-  dim3 grid((unsigned)(items * Hk), B), block(256);
+  dim3 grid((unsigned)(items * Hk), B * num_splits), block(256);
   hipLaunchKernelGGL((paged_attention_tiled_f32_kernel<DV>), grid, block, lds, stream, (const float*)q, q_stride,
                      (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, max_pages, cu_q,
-                     ctx_len, Hq, Hk, page_size, scale, window);
+                     ctx_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml);
   SA_LAUNCH_CHECK();
   return 0;
 }
 
-// float32 attention of every token of the B segments over their cached keys, 64 rows a workgroup.
-// D a multiple of 16 up to 128, page_size a multiple of 4; max_q_len: the longest segment.
+// float32 attention of every token of the B segments (T tokens) over their cached keys, 64 rows a
+// workgroup.  D a multiple of 16 up to 128, page_size a multiple of 4; max_q_len: the longest
+// segment.  num_splits > 1 cuts every tile's key range into that many parts over the grid; part_o
+// [T Hq num_splits, D] and part_ml [T Hq num_splits, 2] (fp32) then take the parts, which a second
+// kernel merges.
 extern "C" int sa_paged_attention_tiled_f32(const void* q, int q_stride, void* out, const void* k_pages,
                                             const void* v_pages, const int* block_table, int max_pages,
-                                            const int* cu_q, const int* ctx_len, int B, int max_q_len, int Hq,
-                                            int Hk, int D, int page_size, float scale, int window,
-                                            hipStream_t stream) {
-  if (B <= 0 || max_q_len <= 0) return 0;
+                                            const int* cu_q, const int* ctx_len, int B, int T, int max_q_len,
+                                            int Hq, int Hk, int D, int page_size, float scale, int window,
+                                            int num_splits, float* part_o, float* part_ml, hipStream_t stream) {
+  if (B <= 0 || max_q_len <= 0 || T <= 0) return 0;
   if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > 128 || (D & 15) || page_size <= 0 || (page_size & 3) ||
-      max_pages <= 0 || (q_stride & 3))
+      max_pages <= 0 || (q_stride & 3) || num_splits < 1 || num_splits > 64)
     return SA_ERR_ARG;
+  if (num_splits > 1 && (!part_o || !part_ml)) return SA_ERR_ARG;
+  int rc = SA_ERR_ARG;
 #define GO(DV)                                                                                                  \
   case DV:                                                                                                      \
-    return launch_tiled<DV>(q, q_stride, out, k_pages, v_pages, block_table, max_pages, cu_q, ctx_len, B,       \
-                            max_q_len, Hq, Hk, page_size, scale, window, stream)
+    rc = launch_tiled<DV>(q, q_stride, out, k_pages, v_pages, block_table, max_pages, cu_q, ctx_len, B,         \
+                          max_q_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml, stream);    \
+    break
   switch (D / 16) {
     GO(1);
     GO(2);
@@ -338,7 +389,11 @@ extern "C" int sa_paged_attention_tiled_f32(const void* q, int q_stride, void* o
     GO(8);
   }
 #undef GO
-  return SA_ERR_ARG;
+  if (rc != 0 || num_splits == 1) return rc;
+  hipLaunchKernelGGL(paged_attention_merge_f32_kernel, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml,
+                     (float*)out, D, num_splits);
+  SA_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int sa_paged_attention_simple(const void* q, int q_stride, void* out, int act_dtype,

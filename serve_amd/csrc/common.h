@@ -91,3 +91,16 @@ __device__ __forceinline__ void sincos_reduced(float x, float* sn, float* cs) {
     hipError_t e__ = hipGetLastError();        \
     if (e__ != hipSuccess) return (int)e__;    \
   } while (0)
+
+// compute units of the current device (asked once per device; 256 if the runtime will not say)
+static inline int compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}

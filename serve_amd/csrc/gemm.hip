@@ -275,14 +275,27 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
     }
 }
 
-// up to this many rows of float32 activations take gemm_nt_rows_kernel (in passes of eight)
-#define ROWS_KERNEL_MAX_M 16
+// Which float32 product a shape takes.  gemm_nt_rows_kernel (passes of eight rows, each reading W
+// again) does about 22 TFLOP/s whatever the shape; the matrix-core kernel takes about 0.078 us per
+// element of K for every round of 128 x 128 tiles over the compute units, however few tiles there
+// are (both measured on an MI355X).  Up to 16 rows always take the first; up to ROWS_KERNEL_MAX_M
+// rows take the one with the smaller estimate (few tiles: a narrow W, decode batches of 17 to 128).
+#define ROWS_KERNEL_MAX_M 128
+static bool rows_kernel_is_faster(int M, int N, int K) {
+  if (M <= 16) return true;
+  if (M > ROWS_KERNEL_MAX_M) return false;
+  const double rows_us = 2.0 * M * N * K / 22e6;
+  const long long tiles = (long long)((N + 127) / 128) * ((M + 127) / 128);
+  const int cus = compute_units();
+  const double mfma_us = 0.078 * K * (double)((tiles + cus - 1) / cus);
+  return rows_us < mfma_us;
+}
 
 extern "C" int sa_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                           int M, int N, int K, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return SA_ERR_ARG;
-  if (a_dtype == SA_F32 && w_dtype == SA_F32 && c_dtype == SA_F32 && M <= ROWS_KERNEL_MAX_M && (K & 3) == 0 &&
+  if (a_dtype == SA_F32 && w_dtype == SA_F32 && c_dtype == SA_F32 && (K & 3) == 0 && rows_kernel_is_faster(M, N, K) &&
       (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
     if (M == 1) return launch_rows<1>(A, W, C, M, N, K, stream);
     if (M == 2) return launch_rows<2>(A, W, C, M, N, K, stream);

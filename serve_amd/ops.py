@@ -227,9 +227,11 @@ def tiled_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_stri
 def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                               v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                               ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int,
-                              scale: float, window: Optional[int]) -> torch.Tensor:
-    """float32 attention of prompt portions: 64 rows (tokens x the query heads of a KV head) a
-    workgroup share the keys and values of their KV head through LDS (fp32 arithmetic on the vector ALU)."""
+                              scale: float, window: Optional[int], num_splits: int = 1) -> torch.Tensor:
+    """float32 attention: 64 rows (tokens x the query heads of a KV head) a workgroup share the keys
+    and values of their KV head through LDS (fp32 arithmetic on the vector ALU).  `num_splits` > 1
+    cuts the key range of every tile into that many parts across workgroups, merged by a second kernel
+    (for single tokens over long contexts, where there are few tiles)."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
     P, Hk, page_size, D = k_pages.shape
     _check(tiled_attention_available(q, k_pages, q_row_stride),
@@ -245,19 +247,25 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
     B = block_table.shape[0]
     _i32(cu_q, B + 1, "cu_q")
     _i32(ctx_len, B, "ctx_len")
-    _check(1 <= max_q_len <= max(T, 1), "max_q_len out of range")
+    _check(1 <= max_q_len <= max(T, 1) and 1 <= num_splits <= 64, "max_q_len / num_splits out of range")
+    part_o = part_ml = None
+    if num_splits > 1:
+        part_o = torch.empty((T * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
     lib = load_library("attention_simple")
     _ret(lib.sa_paged_attention_tiled_f32(
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(max_q_len), c_int(num_heads),
-        c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0), _stream()),
-        "paged_attention_tiled_f32")
+        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(T), c_int(max_q_len),
+        c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0),
+        c_int(num_splits), _ptr(part_o), _ptr(part_ml), _stream()), "paged_attention_tiled_f32")
     return out
 
 
 # rows (tokens x query heads of a KV head) of the longest segment from which the float32 path's tiled
-# attention is taken; below, the one-wave-per-row kernel has nothing to share
+# attention is taken whatever the context; with fewer rows (single tokens) it is taken for contexts from
+# TILED_MIN_CONTEXT on, with the keys cut across workgroups, and the one-wave-per-row kernel below that
 TILED_MIN_ROWS = 16
+TILED_MIN_CONTEXT = 256
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -611,9 +619,17 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
                                  t_end, max_q, num_heads, scale, window, splits, s0, n, in_workgroup=inside)
         return out
     Hk = k_pages.shape[1]
-    if (tiled_attention_available(q, k_pages, q_row_stride)
-            and ctx.max_q_len * (num_heads // Hk) > TILED_MIN_ROWS):
-        return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
-                                         ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window)
+    if tiled_attention_available(q, k_pages, q_row_stride):
+        rows = ctx.max_q_len * (num_heads // Hk)
+        if rows > TILED_MIN_ROWS:
+            return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
+                                             ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window)
+        if ctx.max_ctx_len >= TILED_MIN_CONTEXT:
+            # few rows over many keys: about two workgroups per compute unit, parts of at least 256 keys
+            tiles = ctx.num_segments * Hk
+            splits = max(1, min(64, 2 * compute_units() // max(tiles, 1), ctx.max_ctx_len // 256))
+            return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
+                                             ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window,
+                                             splits)
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                   ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

@@ -263,7 +263,7 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
                                    T, Hq, scale, window)
     elif kernel == "tiled":
         ops.paged_attention_tiled_f32(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
-                                      max(ql for _, ql in segs), Hq, scale, window)
+                                      max(ql for _, ql in segs), Hq, scale, window, splits)
     elif kernel == "dispatch":
         # the way the attention part calls it: the step's facts decide how many launches there are
         from types import SimpleNamespace
@@ -325,6 +325,18 @@ def test_paged_attention_tiled_f32_window_standout_and_poison():
     attention_case("float32", 6, 2, 64, 16, [(0, 90), (200, 40), (77, 3)], seed=19, poison=True, kernel="tiled")
     attention_case("float32", 6, 2, 64, 16, [(150, 40), (300, 2), (64, 64)], seed=20, window=48, poison=True,
                    kernel="tiled")
+
+
+@pytest.mark.parametrize("splits", [2, 3, 7, 64])
+def test_paged_attention_tiled_f32_split_keys(splits):
+    """The key range of every tile cut into parts across workgroups and merged: more parts than blocks
+    of keys (empty parts), rows of a portion that see no key of a part, a window, unowned pages NaN."""
+    segs = [(700, 1), (0, 1), (63, 1), (1300, 1), (129, 1)]
+    attention_case("float32", 8, 2, 64, 16, segs, seed=400 + splits, kernel="tiled", splits=splits, poison=True)
+    attention_case("float32", 3, 1, 48, 8, [(500, 1), (90, 1)], seed=410 + splits, kernel="tiled", splits=splits,
+                   standout=True)
+    attention_case("float32", 4, 2, 32, 8, [(300, 40), (50, 1), (400, 3)], seed=420 + splits, kernel="tiled",
+                   splits=splits, window=100, poison=True)
 
 
 def test_attention_reduces_to_library_routine():

@@ -1,6 +1,7 @@
 """Parts and whole architectures that live in these tests only, registered, built and stepped
 without a change to the framework's files: a layer that keeps a window of keys beside one that
-keeps all (two cache groups); a learned absolute position embedding, a layer arrangement with
+keeps all (two cache groups); a run order that names a layer twice and lets a layer read another
+layer's cache; a learned absolute position embedding, a layer arrangement with
 four norms and a head tied to a tensor of another name; a mixer that caches one latent vector
 per token; a position encoding that the attention kernels do not know.  None of them is a
 model of anyone's: they show what the interfaces carry."""
@@ -117,6 +118,119 @@ def test_windowed_layer_through_the_runner(tmp_path, dtype):
         runner.release(k)
     cache.check_invariants()
     assert cache.free_pages(0) == 40 and cache.free_pages(1) == 40
+
+
+# ---------------------------------------------------------------------------------------------
+# a run order that names a layer twice and lets a layer read another layer's cache
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_run_order_repeats_a_layer_and_shares_a_cache(tmp_path, dtype):
+    """Three layers of weights, four entries in the run order: layer 0, layer 1, layer 0 again (the
+    same weights over a cache layer of its own), then layer 2, whose queries read the keys and
+    values that layer 1 stored and which stores nothing itself.  Three cache layers for four
+    entries.  Portions, single tokens from a graph, two requests beside each other, against the
+    plain parts run in that order."""
+    import serve_amd
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.spec import RunEntry
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    from serve_amd.models.llama import build_llama_spec
+    from serve_amd.weights.loader import write_random_model
+
+    base = dataclasses.replace(util.TINY_C, vocab_size=173, num_hidden_layers=3)
+    order = [RunEntry(0, 0), RunEntry(1, 1), RunEntry(0, 2), RunEntry(2, 1, writes_cache=False)]
+
+    @dataclass(frozen=True)
+    class LoopedConfig:
+        inner: object = base
+        architecture = "ToyLoopedLM"
+
+        def to_hf_dict(self):
+            return dict(self.inner.to_hf_dict(), architectures=[self.architecture])
+
+        @staticmethod
+        def from_hf_dict(d):
+            from serve_amd.config.llama import LlamaConfig
+            return LoopedConfig(LlamaConfig.from_hf_dict(dict(d, architectures=["LlamaForCausalLM"])))
+
+    def build(cfg):
+        return dataclasses.replace(build_llama_spec(cfg.inner), architecture=cfg.architecture, run_order=order)
+
+    serve_amd.register_architecture("ToyLoopedLM", LoopedConfig.from_hf_dict, build)
+    folder = write_random_model(str(tmp_path / "looped"), LoopedConfig(), seed=21, scales=util.SHARP_SCALES)
+    eng = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=8, num_pages=40, max_context=128,
+                                                 max_requests=4, max_tokens_per_step=4096, prefill_chunk=4096))
+    runner, cache = eng.runner, eng.runner.cache
+    assert len(runner.model.cache_requests()) == 3 and len(runner.model.layers) == 3
+
+    # the plain parts in the same order (whole sequences, no cache)
+    w, cfg = util.plain_weights(folder), util.plain_config(folder)
+    Hq, Hk, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], P.head_dim_of(cfg)
+    eps = cfg["rms_norm_eps"]
+
+    def plain(tokens):
+        S = len(tokens)
+        pos = torch.arange(S)
+        table = P.rope_table(pos, P.rope_frequencies(D, cfg["rope_theta"], cfg.get("rope_scaling")))
+        x = w["model.embed_tokens.weight"].double()[torch.as_tensor(tokens)]
+
+        def keys_values(h, layer):
+            p = f"model.layers.{layer}.self_attn."
+            wk = P.permute_rows_for_adjacent_pairs(w[p + "k_proj.weight"].double(), Hk, D)
+            return (P.apply_rope_adjacent((h @ wk.T).view(S, Hk, D), table),
+                    (h @ w[p + "v_proj.weight"].double().T).view(S, Hk, D))
+
+        def block(x, layer, kv=None):
+            p = f"model.layers.{layer}."
+            h = P.rms_norm(x, w[p + "input_layernorm.weight"].double(), eps)
+            k, v = keys_values(h, layer) if kv is None else kv
+            wq = P.permute_rows_for_adjacent_pairs(w[p + "self_attn.q_proj.weight"].double(), Hq, D)
+            q = P.apply_rope_adjacent((h @ wq.T).view(S, Hq, D), table)
+            x = x + P.causal_attention(q, k, v).reshape(S, Hq * D) @ w[p + "self_attn.o_proj.weight"].double().T
+            h2 = P.rms_norm(x, w[p + "post_attention_layernorm.weight"].double(), eps)
+            x = x + P.swiglu(h2, w[p + "mlp.gate_proj.weight"].double(), w[p + "mlp.up_proj.weight"].double(),
+                             w[p + "mlp.down_proj.weight"].double())
+            return x, (k, v)
+
+        x, _ = block(x, 0)
+        x, kv1 = block(x, 1)
+        x, _ = block(x, 0)
+        x, _ = block(x, 2, kv1)
+        x = P.rms_norm(x, w["model.norm.weight"].double(), eps)
+        return x @ P.lm_head_weight(w, cfg).double().T
+
+    rng = random.Random(5)
+    toks = {"a": util.random_tokens(rng, 60, 173), "b": util.random_tokens(rng, 41, 173)}
+    cuts = {"a": [13, 2, 20] + [1] * 25, "b": [30] + [1] * 11}
+    fed = {"a": 0, "b": 0}
+    rows = {"a": [], "b": []}
+    runner.admit("a")
+    step = 0
+    while any(cuts.values()):
+        if step == 1:
+            runner.admit("b")
+        segs = []
+        for k in ("a", "b"):
+            if k in cache and cuts[k]:
+                n = cuts[k].pop(0)
+                segs.append(Segment(k, toks[k][fed[k]: fed[k] + n], list(range(n))))
+                fed[k] += n
+        out = eng.step(segs)
+        at = 0
+        for sg in segs:
+            rows[sg.req_id].append(out[at: at + len(sg.tokens)])
+            at += len(sg.tokens)
+        cache.check_invariants()
+        step += 1
+    assert any(e.graph is not None for e in runner._graphs.values()), "the single tokens were not replayed from a graph"
+    for k in toks:
+        want = plain(toks[k])
+        util.assert_close(torch.cat(rows[k]), want, dtype, f"looped {k}")
+        # the order matters: the llama order of the same weights gives other logits
+        assert (P.forward(toks[k], w, cfg) - want).abs().max().item() > 0.1
+        runner.release(k)
+    cache.check_invariants()
 
 
 # ---------------------------------------------------------------------------------------------

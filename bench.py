@@ -275,8 +275,9 @@ def main() -> int:
     # batch, same bucket of contexts, so the same graph) for at least `--prewarm` seconds, so that a
     # short run measures the device at its running clocks and not the first replays on a cold one
     prewarm_s = 0.0
-    if args.prewarm > 0:
-        n_pre = max(1, min(256, args.context // 4))
+    # (as many steps as leave room for a prompt in the context, beside the head start of the first requests)
+    n_pre = min(256, args.context // 4, args.context - 4 - head_start(engine, args.batch, args.context))
+    if args.prewarm > 0 and n_pre >= 1:
         t0 = time.perf_counter()
         while time.perf_counter() - t0 < args.prewarm:
             decode_run(engine, args.batch, args.context - n_pre - 3 - head_start(engine, args.batch, args.context), 0,

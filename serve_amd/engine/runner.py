@@ -23,6 +23,9 @@ from .batch import Segment, StepLayout, build_step, context_from, plan_step
 
 # padded batch sizes for which decode-only steps are captured into graphs
 GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+# more rows than that are replayed from graphs only where nobody asks for the logits (steps launched
+# ahead of the host, which sample on the device): such a graph keeps no [rows, vocabulary] buffer
+ASYNC_GRAPH_BATCHES = GRAPH_BATCHES + (384, 512)
 
 
 class _GraphEntry:
@@ -102,7 +105,7 @@ class ModelRunner:
         self._graphs = {}
         self._graph_pool = None
         # tokens sampled by the latest decode launch, by row: the next launch may read them here
-        self.sampled = torch.zeros(max(GRAPH_BATCHES[-1], cfg.max_requests), dtype=torch.int32, device=rt.device)
+        self.sampled = torch.zeros(max(ASYNC_GRAPH_BATCHES[-1], cfg.max_requests), dtype=torch.int32, device=rt.device)
         self._row_of = {}
         self._use_graphs = bool(cfg.use_graphs) and model.graph_safe()
         # steps launched ahead of the host need parts that never read back from the device
@@ -148,7 +151,7 @@ class ModelRunner:
         return logits
 
     # -- decode-only steps replayed from HIP graphs ---------------------------------------------------
-    def _decode_core(self, segments: Sequence[Segment], temps=None, keys=None, src_rows=None):
+    def _decode_core(self, segments: Sequence[Segment], temps=None, keys=None, src_rows=None, keep_logits=True):
         """One token per request, sampling included.  The kernel sequence of such a step depends
         only on the padded batch size and on the bucket of the longest context (which fixes the
         attention's key splits), so it is captured once per (batch, bucket) into a HIP graph and
@@ -157,9 +160,10 @@ class ModelRunner:
 
         A row's token id is given by the caller, or (src_rows[i] >= 0) is the token that the
         previous launch sampled into row src_rows[i] of `self.sampled` and that never left the
-        device.  Returns (entry, logits, context lengths)."""
+        device.  Returns (entry, logits, context lengths); without `keep_logits` the logits may be
+        None (more rows than GRAPH_BATCHES holds: the graph then keeps none)."""
         B = len(segments)
-        b_pad = next(b for b in GRAPH_BATCHES if b >= B)
+        b_pad = next(b for b in (GRAPH_BATCHES if keep_logits else ASYNC_GRAPH_BATCHES) if b >= B)
         longest = 1 + max(self.cache.tokens_of(s.req_id) for s in segments)
         bucket = 256
         while bucket < longest:
@@ -204,13 +208,14 @@ class ModelRunner:
             def run():
                 logits = self.model.forward(ctx, self.storage.layers)
                 ops.sample(logits, t_dev, k_dev, self.sampled[:b_pad])
-                return logits
+                # (dropped inside the capture, a large graph's logits go back to the pool the graphs share)
+                return logits if b_pad <= GRAPH_BATCHES[-1] else None
             entry.runs += 1
             logits = run()
             if entry.runs >= 2:
                 # every library is loaded and warm by now: capture for the following steps
                 # all graphs take their intermediate buffers from one pool (they never run side by
-                # side); what a graph keeps for itself is its logits [b_pad, V]
+                # side); what a graph keeps for itself is its logits [b_pad, V], up to 256 rows
                 if self._graph_pool is None:
                     self._graph_pool = torch.cuda.graph_pool_handle()
                 g = torch.cuda.CUDAGraph()
@@ -233,7 +238,7 @@ class ModelRunner:
         return logits, ctx_lens
 
     def can_decode_async(self, n: int) -> bool:
-        return self._use_graphs and 0 < n <= GRAPH_BATCHES[-1]
+        return self._use_graphs and 0 < n <= ASYNC_GRAPH_BATCHES[-1]
 
     def can_launch_ahead(self) -> bool:
         return self._launch_ahead
@@ -250,7 +255,7 @@ class ModelRunner:
             src = [-1 if t is not None else self._row_of[r] for r, t in zip(req_ids, tokens)]
             segments = [Segment(r, [0 if t is None else t], [0]) for r, t in zip(req_ids, tokens)]
             entry, _, ctx_lens = self._decode_core(segments, np.asarray(temperatures, dtype=np.float32),
-                                                   np.asarray(keys, dtype=np.int64), src)
+                                                   np.asarray(keys, dtype=np.int64), src, keep_logits=False)
             self._row_of = {r: i for i, r in enumerate(req_ids)}
             host = entry.host_tokens[entry.launches & 1]
             entry.launches += 1

@@ -121,6 +121,33 @@ def test_graph_decode_of_many_requests_across_a_context_bucket(tmp_path, name, c
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_more_than_256_requests_decode_from_a_graph_that_keeps_no_logits(tmp_path, dtype):
+    """300 requests generate through the entry point, sampled on the device: their decode steps have
+    more rows than the graphs with logits take and are replayed from a graph of 384 rows that keeps
+    none; the tokens are the plain model's."""
+    from serve_amd.engine.engine import Request
+    folder = util.make_folder(tmp_path, "AS")
+    vocab = util.tiny_config("AS").vocab_size
+    rng = random.Random(31)
+    count, new = 300, 7
+    prompts = [util.random_tokens(rng, rng.randrange(3, 9), vocab) for _ in range(count)]
+    engine = make_engine(folder, dtype, page_size=8, num_pages=count * 3, max_context=64, max_requests=count,
+                         max_tokens_per_step=4096, prefill_chunk=64, seed=SEED)
+    log = []
+    temps = [0.0 if i % 3 else 0.7 for i in range(count)]
+    out = engine.generate([Request(torch.tensor(p), len(p), new) for p in prompts], temperature=temps, step_log=log)
+    big = [st for st in log if len(st["requests"]) > 256 and set(st["counts"]) == {1}]
+    assert len(big) >= 4, "no decode steps of more than 256 requests were run"
+    entry = engine.runner._graphs.get((384, 256))
+    assert entry is not None and entry.graph is not None and entry.logits is None
+    assert all(o.error is None and len(o.generated_tokens) == new for o in out)
+    for i in list(range(0, count, 13)) + [count - 1]:
+        check_tokens(folder, prompts[i], out[i].generated_tokens.tolist(), dtype, f"request {i} of {count}",
+                     temperature=temps[i], rid=i)
+    engine.runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_stop_tokens_end_a_request_and_free_its_pages(tmp_path, dtype):
     """A token id that the greedy continuation of request 1 contains ends it there (the id stays
     in its tokens); requests whose continuation does not contain it are unchanged; its pages and

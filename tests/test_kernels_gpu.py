@@ -73,8 +73,10 @@ def test_add_rmsnorm(dtype, d, eps):
                                    # up to 16 rows of float32 with K % 4 == 0: the weight-streaming kernel
                                    (1, 2049, 2048), (8, 509, 1100), (16, 130, 8192), (5, 8200, 36), (2, 3, 4),
                                    (9, 8193, 1028),
-                                   # more rows with K % 4 == 0: the matrix cores' float32 instruction
-                                   (200, 300, 2048), (129, 257, 64), (1000, 128, 512), (33, 40, 4), (128, 128, 16)])
+                                   # more rows with K % 4 == 0: the matrix cores' float32 instruction, or (up to
+                                   # 128 rows, where its tiles would be few) the weight-streaming kernel again
+                                   (200, 300, 2048), (129, 257, 64), (1000, 128, 512), (33, 40, 4), (128, 128, 16),
+                                   (100, 2048, 512), (40, 66000, 64)])
 def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
     from serve_amd import ops
     a = rnd((M, K), DT[a_dt], 4)

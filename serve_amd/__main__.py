@@ -20,9 +20,10 @@ def _generate(argv) -> int:
     ap = argparse.ArgumentParser(prog="python -m serve_amd generate")
     src = ap.add_mutually_exclusive_group(required=True)
     src.add_argument("--model", help="model folder (config.json + model.safetensors)")
-    src.add_argument("--shape", help="a named shape with random weights drawn from --seed (tiny, tiny-a, tiny-b, "
+    src.add_argument("--shape", "--preset", dest="shape", help="a named shape with random weights drawn from --seed (tiny, tiny-a, tiny-b, "
                      "llama-1b, llama-3b, llama-8b)")
-    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--dtype", type=dtype_name, choices=["bfloat16", "float32"], default="bfloat16",
+                    help="bfloat16 (or bf16), float32 (or fp32)")
     ap.add_argument("--prompt-ids", help="file with one prompt a line: JSON list or blank-separated token ids "
                     "(default: standard input)")
     ap.add_argument("--random-prompts", metavar="N:LEN", help="N prompts of LEN uniform random token ids "
@@ -94,7 +95,7 @@ def _random_model(argv) -> int:
     ap = argparse.ArgumentParser(prog="python -m serve_amd random-model")
     ap.add_argument("--out", required=True, help="folder to write config.json and model.safetensors into")
     g = ap.add_mutually_exclusive_group(required=True)
-    g.add_argument("--shape", help="a named shape (tiny, tiny-a, tiny-b, llama-1b, llama-3b, llama-8b)")
+    g.add_argument("--shape", "--preset", dest="shape", help="a named shape (tiny, tiny-a, tiny-b, llama-1b, llama-3b, llama-8b)")
     g.add_argument("--config", help="a config.json to take the sizes from")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--weight-dtype", choices=["bfloat16", "float32"], default="bfloat16",
@@ -118,6 +119,11 @@ def _random_model(argv) -> int:
     return 0
 
 
+def dtype_name(text: str) -> str:
+    """The long name of a dtype given by either name."""
+    return {"bf16": "bfloat16", "fp32": "float32"}.get(text, text)
+
+
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     commands = {"generate": _generate, "random-model": _random_model}
@@ -128,7 +134,7 @@ def main(argv=None) -> int:
     if cmd == "replay":
         from .engine.replay import main as replay_main
         return replay_main(rest)
-    if cmd == "benchmark":
+    if cmd in ("benchmark", "bench"):
         from .benchmark import main as bench_main
         return bench_main(rest)
     if cmd not in commands:

@@ -74,8 +74,10 @@ def main(argv=None) -> int:
     ap.add_argument("--profile-only", action="store_true", help="skip the timed run (serve/benchmark.py:69)")
     src = ap.add_mutually_exclusive_group()
     src.add_argument("--model", help="model folder (config.json + model.safetensors)")
-    src.add_argument("--shape", choices=sorted(SHAPES), default="llama-1b", help="named shape, random weights")
-    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    src.add_argument("--shape", "--preset", dest="shape", choices=sorted(SHAPES), default="llama-1b",
+                     help="named shape, random weights")
+    ap.add_argument("--dtype", type=lambda t: {"bf16": "bfloat16", "fp32": "float32"}.get(t, t),
+                    choices=["bfloat16", "float32"], default="bfloat16", help="bfloat16 (or bf16), float32 (or fp32)")
     ap.add_argument("--input-length", type=int, default=256)
     ap.add_argument("--output-length", type=int, default=256)
     ap.add_argument("--num-sequences", type=int, default=2000)

@@ -278,3 +278,19 @@ def test_rotary_part_refuses_contexts_beyond_its_kernels_angles():
     part.load({}, Runtime(torch.device("cpu"), torch.bfloat16, max_context=1_000_000))
     part.load({}, Runtime(torch.device("cpu"), torch.float32, max_context=8_000_000))
     assert part.rotary().rot_dim == 64 and not part.rotary().adjacent_pairs
+
+
+def test_command_line_writes_a_random_model_and_knows_the_short_names(tmp_path):
+    """`random-model` needs no GPU: a folder from a named shape (`--preset` is another name of
+    `--shape`), readable by the loader's own reader; `bf16` and `fp32` are other names of the dtypes."""
+    from serve_amd.__main__ import dtype_name, main
+    from serve_amd.registry import load_config
+    from serve_amd.weights.safetensors_io import CheckpointReader
+    assert dtype_name("bf16") == "bfloat16" and dtype_name("fp32") == "float32" and dtype_name("float32") == "float32"
+    out = str(tmp_path / "m")
+    assert main(["random-model", "--preset", "tiny-a", "--out", out, "--seed", "4", "--weight-dtype", "float32"]) == 0
+    _, cfg = load_config(out)
+    assert cfg.hidden_size == 64 and cfg.num_hidden_layers == 2
+    reader = CheckpointReader(out)
+    assert "model.embed_tokens.weight" in reader.names()
+    assert main(["no-such-command"]) == 2

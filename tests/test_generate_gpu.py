@@ -44,19 +44,28 @@ def test_greedy_generation_tiny_a_whole_prompts(tmp_path):
     model.runner.cache.check_invariants()
 
 
+@pytest.mark.parametrize("vocab", [509, 512])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sampled_generation_tiny_b_chunked_beside_decodes(tmp_path, dtype):
+def test_sampled_generation_tiny_b_chunked_beside_decodes(tmp_path, dtype, vocab):
     """Tiny B's workload: prompts of 5, 17, 30 and 2 tokens prefilled in chunks of 8 beside decoding
     requests, 6 draws at temperature 0.8 with a fixed sampler seed, page size 8.  Each draw must be
     the plain sampler's draw from the engine's own logits path: teacher-forced on the engine's
-    tokens, the plain logits give the same token unless two scores are within the dtype's error."""
+    tokens, the plain logits give the same token unless two scores are within the dtype's error.
+    With the vocabulary of 512 the configuration is specified with (the named shape tiny-b), and with
+    the 509 of the other tests, which is no power of two."""
+    from serve_amd.benchmark import SHAPES
     from serve_amd.config.engine import EngineConfig
     from serve_amd.engine.engine import Engine, Request
-    folder = util.make_folder(tmp_path, "B")
+    from serve_amd.weights.loader import write_random_model
+    if vocab == 512:
+        assert SHAPES["tiny-b"].vocab_size == 512
+        folder = write_random_model(str(tmp_path / "tiny_b_512"), SHAPES["tiny-b"], 1)
+    else:
+        folder = util.make_folder(tmp_path, "B")
     eng = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=8, num_pages=24, max_context=64,
                                                  max_requests=4, prefill_chunk=8, max_tokens_per_step=12, seed=77))
     rng = random.Random(1)
-    prompts = [util.random_tokens(rng, n, 509) for n in (5, 17, 30, 2)]
+    prompts = [util.random_tokens(rng, n, vocab) for n in (5, 17, 30, 2)]
     out = eng.generate([Request(torch.tensor(p), len(p), 6) for p in prompts], temperature=0.8)
     w, cfg = util.plain_weights(folder), util.plain_config(folder)
     margin = 1e-4 if dtype == "float32" else 5e-2
@@ -66,7 +75,7 @@ def test_sampled_generation_tiny_b_chunked_beside_decodes(tmp_path, dtype):
         seq = list(p)
         for i, t in enumerate(got):
             logits = llama_plain.forward(seq, w, cfg)[-1]
-            noise = llama_plain.exponential_noise(77, rid, i, 509).double()
+            noise = llama_plain.exponential_noise(77, rid, i, vocab).double()
             score = logits / 0.8 - noise.log()
             assert score.max() - score[t] <= margin, f"request {rid} token {i}: {t} is not the draw"
             seq.append(t)

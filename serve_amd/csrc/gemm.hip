@@ -181,6 +181,7 @@ __device__ __forceinline__ float4 load4f(const bf16_t* p) {
 #define MF_BM 128
 #define MF_BN 128
 #define MF_BK 16
+#define MF_FLUSH 32                // slices of K (512 terms) summed in one accumulator before they join the total
 
 template <typename TA, typename TW, typename TC>
 __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
@@ -230,13 +231,16 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
       w[0] = rw[j].x; w[1] = rw[j].y; w[2] = rw[j].z; w[3] = rw[j].w;
     }
   };
-  floatx16_t acc[2][2];
+  // two levels of sums: `acc` takes MF_FLUSH slices of K and is then added to `total`, so that no sum
+  // runs over more than a few hundred terms in one accumulator (the rounding of a float32 sum grows
+  // with its length)
+  floatx16_t acc[2][2], total[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = total[i][j][e] = 0.f;
 
   const int nslices = (K + MF_BK - 1) / MF_BK;
   fetch(0);
@@ -260,6 +264,16 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
         for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], w[j], acc[i][j], 0, 0, 0);
     }
     if (s + 1 < nslices) stash(b ^ 1);
+    if ((s & (MF_FLUSH - 1)) == MF_FLUSH - 1 || s + 1 == nslices) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          total[i][j] += acc[i][j];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        }
+    }
     __syncthreads();
   }
 #pragma unroll
@@ -270,7 +284,7 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * kh + (e & 3);
-        if (m < M && n < N) C[(size_t)m * N + n] = from_float<TC>(acc[i][j][e]);
+        if (m < M && n < N) C[(size_t)m * N + n] = from_float<TC>(total[i][j][e]);
       }
     }
 }

@@ -543,28 +543,37 @@ static bool takes_skinny(int M, int N, const QkvRopeArgs& qa) {
 template <typename TC, int EPI>
 static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                     const QkvRopeArgs& qa, hipStream_t stream) {
-  // 16-row tiles of activations per pass: up to 128 rows in one pass (more rows: more passes, each
-  // streaming the weights again, which the caller avoids)
-  const int mt = M > 64 ? 8 : (M > 32 ? 4 : (M > 16 ? 2 : 1));
+  // 16-row tiles of activations per pass, as many as the rows need: up to 128 rows in one pass
+  // (more rows: more passes, each streaming the weights again, which the caller avoids)
+  const int mt = min(8, (M + 15) / 16);
 #define GO(RT, MT, NR, KH) \
   return launch_mid<RT, MT, NR, KH, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
+  // up to four tiles: a workgroup shape for one, for two, and for three or four tiles
 #define GO3(RT, NR1, KH1, NR2, KH2, NR4, KH4) \
   do {                                         \
     if (mt == 1) GO(RT, 1, NR1, KH1);          \
     if (mt == 2) GO(RT, 2, NR2, KH2);          \
+    if (mt == 3) GO(RT, 3, NR4, KH4);          \
     if (mt == 4) GO(RT, 4, NR4, KH4);          \
   } while (0)
-  // (with eight tiles a workgroup has 512 threads or more: fewer would hold too many activation
-  // segments each on their way into LDS)
+  // five to eight tiles: one shape (a workgroup then has 512 threads or more: fewer would hold too
+  // many activation segments each on their way into LDS)
+#define GO8(RT, NR, KH)                   \
+  do {                                    \
+    if (mt == 5) GO(RT, 5, NR, KH);       \
+    if (mt == 6) GO(RT, 6, NR, KH);       \
+    if (mt == 7) GO(RT, 7, NR, KH);       \
+    GO(RT, 8, NR, KH);                    \
+  } while (0)
   if constexpr (EPI == EPI_PLAIN) {
     if (N < 8192) {
       GO3(1, 2, 4, 2, 4, 2, 4);                // 32 weight rows a workgroup, K cut four ways inside it
-      GO(1, 8, MID8_PLAIN_NR, MID8_PLAIN_KH);
+      GO8(1, MID8_PLAIN_NR, MID8_PLAIN_KH);
     }
     if (M <= 8) GO(1, 1, 4, 2);                // the head: 64 weight rows, or 128 with two passes' worth of rows
     if (M <= 32) GO(1, 2, 8, 2);
     if (M <= 64) GO(1, 4, 8, 2);
-    GO(1, 8, MID8_HEAD_NR, MID8_HEAD_KH);
+    GO8(1, MID8_HEAD_NR, MID8_HEAD_KH);
   }
   if constexpr (EPI == EPI_QKV_ROPE) {
     const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
@@ -575,17 +584,18 @@ static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, 
       GO(1, 4, 1, 8);
     }
     GO3(1, 2, 2, 2, 4, 2, 4);                    // two tiles
-    GO(1, 8, 2, 4);
+    GO8(1, 2, 4);
   }
   if constexpr (EPI == EPI_SWIGLU) {
     const int tiles = (N + 15) / 16;             // N: rows of the gate (and of the up) matrix
     if (tiles < 768) {
       GO3(2, 1, 8, 2, 2, 2, 2);                  // 32 to 64 weight rows a workgroup
-      GO(2, 8, MID8_SWIGLU_NR, MID8_SWIGLU_KH);
+      GO8(2, MID8_SWIGLU_NR, MID8_SWIGLU_KH);
     }
     GO3(2, 4, 2, 4, 2, 4, 2);                    // 128
-    GO(2, 8, MID8_SWIGLU_NR, MID8_SWIGLU_KH);
+    GO8(2, MID8_SWIGLU_NR, MID8_SWIGLU_KH);
   }
+#undef GO8
 #undef GO3
 #undef GO
   return SA_ERR_ARG;

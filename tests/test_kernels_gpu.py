@@ -539,9 +539,9 @@ def test_prompt_attention_long_prompts_windows_and_split_keys(Hq, Hk, D, ps):
 @pytest.mark.parametrize("M,N,K", [(1, 70, 40), (3, 64, 64), (8, 3072, 2048), (16, 509, 96), (17, 130, 104),
                                    (33, 2048, 8192), (64, 8200, 256), (100, 77, 1024), (8, 128256 // 8, 192),
                                    (2, 8200, 72), (5, 9001, 64), (24, 8193, 520), (12, 520, 1032),
-                                   # 65 to 128 rows: eight 16-row tiles a pass; more rows: several passes
+                                   # 65 to 128 rows: five to eight 16-row tiles a pass; more rows: several passes
                                    (65, 2048, 2048), (100, 333, 264), (128, 8200, 520), (127, 3072, 2048),
-                                   (200, 130, 512)])
+                                   (90, 2048, 520), (90, 8200, 264), (45, 8200, 136), (200, 130, 512)])
 def test_gemm_bf16_skinny(c_dt, M, N, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 4)
@@ -562,7 +562,9 @@ def test_gemm_bf16_skinny(c_dt, M, N, K):
                                    # many rows of weights: 128 of them a workgroup
                                    (1, 12300, 64), (7, 12300, 264), (24, 14336, 128), (64, 12296, 72),
                                    # 65 to 128 rows
-                                   (65, 1000, 96), (128, 8192, 2048), (97, 12296, 136), (113, 520, 1032)])
+                                   (65, 1000, 96), (128, 8192, 2048), (97, 12296, 136), (113, 520, 1032),
+                                   # three and six tiles
+                                   (40, 1000, 96), (88, 12300, 136), (88, 520, 264), (35, 12300, 72)])
 def test_swiglu_bf16(M, I, K):
     from serve_amd import ops
     a = rnd((M, K), torch.bfloat16, 6)
@@ -637,7 +639,7 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
                                              (64, 28, 2, 128, 16, 264), (3, 60, 4, 64, 16, 64),
                                              # 65 to 128 rows
                                              (65, 32, 8, 64, 16, 2048), (128, 3, 1, 96, 16, 72), (100, 24, 8, 128, 16, 264),
-                                             (77, 4, 2, 16, 8, 40)])
+                                             (77, 4, 2, 16, 8, 40), (90, 24, 8, 128, 16, 136), (110, 28, 2, 128, 16, 72)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
     P = 7 if M <= 64 else 20

@@ -83,10 +83,11 @@ def test_many_decoders_beside_prompt_portions(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,count", [("AS", 8), ("BS", 17), ("CS", 64), ("B32", 5), ("AS", 130), ("CS", 100)])
+@pytest.mark.parametrize("name,count", [("AS", 8), ("BS", 17), ("CS", 64), ("B32", 5), ("AS", 130), ("CS", 100),
+                                        ("BS", 44), ("AS", 75), ("CS", 90)])
 def test_graph_decode_of_many_requests_across_a_context_bucket(tmp_path, name, count, dtype):
     """`count` requests are decoded one token a step for 45 steps while their contexts pass 256
-    tokens: the steps are replayed from graphs of the padded batch (8, 32, 64, 128, 256) for the buckets up
+    tokens: the steps are replayed from graphs of the padded batch (8, 32, 64, 112, 256) for the buckets up
     to 256 and up to 512 keys, and every logit of every step is compared with the plain model."""
     from serve_amd.engine.batch import Segment
     folder = util.make_folder(tmp_path, name)
@@ -108,7 +109,8 @@ def test_graph_decode_of_many_requests_across_a_context_bucket(tmp_path, name, c
         assert logits.shape == (count, vocab)
         for i in range(count):
             got[i].append(logits[i])
-    b_pad = next(b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b >= count)
+    from serve_amd.engine.runner import GRAPH_BATCHES
+    b_pad = next(b for b in GRAPH_BATCHES if b >= count)
     for bucket in (256, 512):
         entry = runner._graphs.get((b_pad, bucket))
         assert entry is not None and entry.graph is not None, f"no graph was replayed for {(b_pad, bucket)}"

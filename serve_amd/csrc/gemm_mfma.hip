@@ -579,8 +579,9 @@ static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, 
     const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
     if (tiles < 256) {
       GO3(1, 1, 8, 1, 8, 1, 8);                  // one 16-row tile a workgroup, K cut eight ways
-      // more than 64 rows: two passes of 64 (the second finds the weights in L2) fill the chip
+      // more than 64 rows: two passes of 48 or 64 (the second finds the weights in L2) fill the chip
       // better than one pass with half as many workgroups (about 3 us less at 128 rows, 1B shape)
+      if (mt <= 6) GO(1, 3, 1, 8);
       GO(1, 4, 1, 8);
     }
     GO3(1, 2, 2, 2, 4, 2, 4);                    // two tiles

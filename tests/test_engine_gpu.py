@@ -256,7 +256,7 @@ def test_random_configurations_random_cuts(tmp_path, seed):
             cuts.shuffle(order)
             segs = []
             for i in order:
-                n = min(lengths[i] - at[i], cuts.choice([1, 1, 2, 3, 17, 64, 130, 300]))
+                n = min(lengths[i] - at[i], cuts.choice([1, 1, 2, 3, 17, 40, 64, 75, 90, 110, 130, 300]))
                 segs.append(Segment(i, tokens[i][at[i]: at[i] + n], list(range(n))))
                 at[i] += n
             if not segs:

@@ -578,9 +578,11 @@ static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, 
   if constexpr (EPI == EPI_QKV_ROPE) {
     const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
     if (tiles < 256) {
-      GO3(1, 1, 8, 1, 8, 1, 8);                  // one 16-row tile a workgroup, K cut eight ways
-      // more than 64 rows: two passes of 48 or 64 (the second finds the weights in L2) fill the chip
-      // better than one pass with half as many workgroups (about 3 us less at 128 rows, 1B shape)
+      // one 16-row tile a workgroup, K cut eight ways.  From 49 rows on two passes of half the rows
+      // (the second finds the weights in L2) fill the chip better than one pass with half as many
+      // workgroups (about 3 us less at 128 rows, 1 us at 64, 1B shape)
+      if (mt == 4) GO(1, 2, 1, 8);
+      GO3(1, 1, 8, 1, 8, 1, 8);
       if (mt <= 6) GO(1, 3, 1, 8);
       GO(1, 4, 1, 8);
     }

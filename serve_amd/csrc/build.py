@@ -43,7 +43,10 @@ SOURCES: Dict[str, str] = {
     "gemm_mfma": "gemm_mfma.hip",
     "attention_mfma": "attention_mfma.hip",
     "membench": "membench.hip",
+    "blaslt": "blaslt.hip",
 }
+# what a library is linked with beside the HIP runtime
+LINK: Dict[str, List[str]] = {"blaslt.hip": ["-lhipblaslt"]}
 
 # variants that are compiled with defines: library name -> list of define sets
 VARIANTS: Dict[str, List[Dict[str, object]]] = {
@@ -99,7 +102,7 @@ def _key(source: str, defines: Tuple[Tuple[str, str], ...]) -> str:
     for name in [source] + HEADERS + OWN_HEADERS.get(source, []):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + LINK.get(source, [])).encode())
     h.update(repr(defines).encode())
     return h.hexdigest()[:16]
 
@@ -150,7 +153,7 @@ def compile_library(name: str, defines: Optional[Dict[str, object]] = None, forc
                         pass
             tmp = out + f".tmp{os.getpid()}"
             cmd = [hipcc] + FLAGS + [f"-D{k}={v}" for k, v in sorted((defines or {}).items())]
-            cmd += ["-I", CSRC, os.path.join(CSRC, SOURCES[name]), "-o", tmp]
+            cmd += ["-I", CSRC, os.path.join(CSRC, SOURCES[name]), "-o", tmp] + LINK.get(SOURCES[name], [])
             env = dict(os.environ)
             # hipcc wants a writable HOME / temp folder for its intermediate files
             if not os.access(env.get("HOME", "/nonexistent"), os.W_OK):

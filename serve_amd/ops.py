@@ -391,18 +391,46 @@ def split_k_parts(M: int, N: int, K: int) -> int:
     return parts
 
 
+BLASLT_WORKSPACE_BYTES = 64 << 20
+_BLASLT_WORKSPACE = {}
+
+
+def blaslt_workspace(device) -> torch.Tensor:
+    """The scratch memory of the BLAS library's products, one buffer per device (the products run
+    in one stream).  Made at the first call: the parts ask for it when they load, so that it
+    does not come out of the memory pool of a graph capture."""
+    dev = torch.device(device)
+    key = dev.index if dev.index is not None else torch.cuda.current_device()
+    ws = _BLASLT_WORKSPACE.get(key)
+    if ws is None:
+        ws = _BLASLT_WORKSPACE[key] = torch.empty(BLASLT_WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
+    return ws
+
+
+def gemm_bf16_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = a @ w^T by the BLAS library (hipBLASLt, called directly: the descriptors and the
+    algorithm of a shape are kept after its first call, so a call costs the host a few
+    microseconds).  bf16 operands, bf16 or fp32 output."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _check(w.shape == (N, K) and out.shape == (M, N), "gemm_bf16_library: shapes do not match")
+    _check(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in (torch.bfloat16, torch.float32)
+           and _aligned16(a, w, out), "gemm_bf16_library needs bf16 operands, a bf16 or fp32 result and 16-byte alignment")
+    ws = blaslt_workspace(a.device)
+    lib = load_library("blaslt")
+    _ret(lib.sa_blaslt_mm(_ptr(a), _ptr(w), _ptr(out), c_int(_code(out)), c_int(M), c_int(N), c_int(K), _ptr(ws),
+                          ctypes.c_size_t(ws.numel()), _stream()), "gemm_bf16_library")
+    return out
+
+
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """bf16 product: the weight-streaming kernels for few rows, the BLAS library for many (the
     reference leaves all of its products to the library, serve/model.py:80-82,95,97,159); both
     write bf16 or fp32."""
     if a.shape[0] <= SKINNY_MAX_ROWS and not (a.shape[0] > 64 and w.shape[0] >= WIDE_OUTPUT):
         return gemm_bf16_skinny(a, w, out)
-    _dev(a, w, out)
-    if out.dtype == torch.bfloat16:
-        torch.mm(a, w.t(), out=out)
-    else:
-        torch.mm(a, w.t(), out_dtype=out.dtype, out=out)
-    return out
+    return gemm_bf16_library(a, w, out)
 
 
 def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

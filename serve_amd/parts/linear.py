@@ -6,7 +6,8 @@ Which kernel runs is decided here and nowhere else:
 * float32 activations or weights -> the fp32 vector-ALU product (`ops.gemm_nt`): the true
   32-bit path, also taken for weights a checkpoint stores in 32-bit;
 * bfloat16 with few rows -> the weight-streaming MFMA kernel (`ops.gemm_bf16_skinny`);
-* bfloat16 with many rows -> the BLAS library, as the reference does for all of its products.
+* bfloat16 with many rows -> the BLAS library (`ops.gemm_bf16_library`), as the reference does for all of
+  its products.
 """
 from __future__ import annotations
 

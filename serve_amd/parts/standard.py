@@ -17,6 +17,13 @@ from .base import (LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime
 from .linear import linear
 
 
+def _prepare_products(rt: Runtime, weight: torch.Tensor) -> None:
+    """What the products over `weight` need beside their operands, made when a part loads and not
+    at its first step (which may run inside a graph capture): the library's scratch memory."""
+    if weight.is_cuda and weight.dtype == torch.bfloat16 and rt.dtype == torch.bfloat16:
+        ops.blaslt_workspace(weight.device)
+
+
 # ---------------------------------------------------------------------------------------------
 # norm
 # ---------------------------------------------------------------------------------------------
@@ -149,6 +156,7 @@ class GQAAttention(Part):
         self.wqkv = torch.cat([p.to(dt) for p in parts], dim=0).contiguous()
         self.wq = self.wqkv[: self.num_heads * self.head_dim]
         self.wo = tensors["o_proj.weight"]
+        _prepare_products(rt, self.wqkv)
         self.position.load({}, rt)
         self._no_freq = torch.empty(0, dtype=torch.float32, device=rt.device)
 
@@ -213,6 +221,7 @@ class SwiGLU(Part):
         dt = g.dtype if g.dtype == u.dtype else torch.float32
         self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
+        _prepare_products(rt, self.w_down)
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         a = self.rt.empty((h.shape[0], self.intermediate_size))
@@ -272,6 +281,7 @@ class LinearHead(Part):
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         self.weight = tensors["weight"]
+        _prepare_products(rt, self.weight)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return linear(h, self.weight, out_dtype=torch.float32)

@@ -671,6 +671,24 @@ def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     assert not ops.qkv_rope_available(h, w, k1, 24, 24, False) and not ops.qkv_rope_available(h, w, k1, D, D, True)
 
 
+@pytest.mark.parametrize("c_dt", ["bfloat16", "float32"])
+@pytest.mark.parametrize("M,N,K", [(129, 2048, 2048), (576, 3072, 2048), (2048, 520, 264), (300, 8200, 1032),
+                                   (1000, 77, 8192), (130, 16032, 72), (4096, 2048, 8192)])
+def test_gemm_bf16_library(c_dt, M, N, K):
+    """The library's product, called directly with kept plans: twice per shape (the second call finds
+    the plan of the first), against fp64."""
+    from serve_amd import ops
+    a = rnd((M, K), torch.bfloat16, 14)
+    w = rnd((N, K), torch.bfloat16, 15, 0.05)
+    want = a.double() @ w.double().T
+    for _ in range(2):
+        out = torch.full((M, N), float("nan"), dtype=DT[c_dt], device=DEV)
+        ops.gemm_bf16_library(a, w, out)
+        torch.testing.assert_close(out.double(), want, atol=2e-2 + 1e-3 * K ** 0.5, rtol=1e-2)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_bf16_library(a.float(), w, out)
+
+
 def test_memory_ceiling_kernels_copy_and_refuse():
     """The plain read and copy kernels of the measurement program: the copy is exact for sizes that
     are no multiple of the grid, misaligned or ragged buffers are refused."""

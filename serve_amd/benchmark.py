@@ -92,7 +92,10 @@ def main(argv=None) -> int:
     ap.add_argument("--max-context", type=int, default=2048, help="serve/model.py:32")
     ap.add_argument("--max-requests", type=int, default=2048, help="requests live at a time at most; the reference "
                     "admits by cache capacity alone (serve/run.py:267-280)")
-    ap.add_argument("--max-tokens-per-step", type=int, default=2048, help="serve/run.py:265")
+    ap.add_argument("--max-tokens-per-step", type=int, default=None,
+                    help="tokens of a step, single decoded tokens and prompt portions together; default: 2048 + "
+                         "--max-requests, since the reference prefills up to 2,048 prompt tokens a step "
+                         "(serve/run.py:265) beside decode steps of their own")
     ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")
     ap.add_argument("--admit-interval", type=int, default=1, help="admit new requests at most every N steps while "
@@ -102,7 +105,8 @@ def main(argv=None) -> int:
     from .engine.engine import Engine
     cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, memory_fraction=args.memory_fraction,
                        max_context=args.max_context, max_requests=args.max_requests,
-                       max_tokens_per_step=args.max_tokens_per_step, prefill_chunk=args.prefill_chunk,
+                       max_tokens_per_step=args.max_tokens_per_step or 2048 + args.max_requests,
+                       prefill_chunk=args.prefill_chunk,
                        admission=args.admission, admit_interval=args.admit_interval, seed=args.seed)
     print(f"loading model {args.model or args.shape}...")
     if args.model:

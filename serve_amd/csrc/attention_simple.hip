@@ -21,7 +21,8 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const TA* __restrict__ q, int q_stride, TA* __restrict__ out, const TC* __restrict__ k_pages,
     const TC* __restrict__ v_pages, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ seg_of_token,
-    int Hq, int Hk, int D, int page_size, float scale, int window, int t0) {
+    int Hq, int Hk, int D, int page_size, float scale, int window, int t0, int num_splits,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
   __shared__ float qs[SA_MAX_D];
   __shared__ float ps[SA_WAVE];
   __shared__ int vbase_page[SA_WAVE];
@@ -42,7 +43,15 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
 
   int lo = 0;
   if (window > 0 && qpos - window + 1 > 0) lo = qpos - window + 1;
-  const int hi = qpos;  // inclusive
+  int hi = qpos;  // inclusive
+  if (num_splits > 1) {
+    // blockIdx.z takes its share of the chunks of 64 keys (it may be empty: then m stays -inf)
+    const int chunks = (hi - lo + SA_WAVE) / SA_WAVE;
+    const int per = (chunks + num_splits - 1) / num_splits;
+    const int first = lo + (int)blockIdx.z * per * SA_WAVE;
+    hi = min(hi, first + per * SA_WAVE - 1);
+    lo = first;
+  }
 
   float m = -INFINITY, l = 0.f;
   float acc[SA_MAX_D / SA_WAVE];
@@ -84,6 +93,20 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
       }
     }
     __syncthreads();
+  }
+  if (num_splits > 1) {
+    // unnormalised sums with their maximum and weight: merged by paged_attention_merge_f32_kernel
+    const size_t slot = ((size_t)t * Hq + h) * num_splits + blockIdx.z;
+#pragma unroll
+    for (int a = 0; a < SA_MAX_D / SA_WAVE; ++a) {
+      const int i = lane + a * SA_WAVE;
+      if (i < D) part_o[slot * D + i] = acc[a];
+    }
+    if (lane == 0) {
+      part_ml[slot * 2] = m;
+      part_ml[slot * 2 + 1] = l;
+    }
+    return;
   }
   const float inv_l = 1.f / l;
   TA* orow = out + (size_t)t * Hq * D + (size_t)h * D;
@@ -401,25 +424,34 @@ extern "C" int sa_paged_attention_simple(const void* q, int q_stride, void* out,
                                          const int* block_table, int max_pages, const int* cu_q,
                                          const int* ctx_len, const int* seg_of_token, int T, int Hq,
                                          int Hk, int D, int page_size, float scale, int window,
-                                         hipStream_t stream) {
+                                         int num_splits, float* part_o, float* part_ml, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > SA_MAX_D || page_size <= 0 || max_pages <= 0)
+  if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > SA_MAX_D || page_size <= 0 || max_pages <= 0 ||
+      num_splits < 1 || num_splits > 64)
     return SA_ERR_ARG;
+  // the key range of every (token, head) cut into num_splits parts over the grid (float32 only):
+  // part_o [T Hq num_splits, D] and part_ml [T Hq num_splits, 2] take the parts, a second kernel merges them
+  if (num_splits > 1 && (!part_o || !part_ml || act_dtype != SA_F32)) return SA_ERR_ARG;
   if (T > 65535 * 16) return SA_ERR_ARG;
   // grid.y is limited to 65535: long steps are launched in slices of tokens
   const int slice = 32768;
   for (int t0 = 0; t0 < T; t0 += slice) {
     const int n = T - t0 < slice ? T - t0 : slice;
-    dim3 grid(Hq, n), block(SA_WAVE);
+    dim3 grid(Hq, n, num_splits), block(SA_WAVE);
 #define GO(TA, TC)                                                                                   \
   hipLaunchKernelGGL((paged_attention_simple_kernel<TA, TC>), grid, block, 0, stream,                \
                      (const TA*)q, q_stride, (TA*)out, (const TC*)k_pages, (const TC*)v_pages,       \
                      block_table, max_pages, cu_q, ctx_len, seg_of_token, Hq, Hk, D, page_size,     \
-                     scale, window, t0)
+                     scale, window, t0, num_splits, part_o, part_ml)
     if (act_dtype == SA_F32 && cache_dtype == SA_F32) GO(float, float);
     else if (act_dtype == SA_BF16 && cache_dtype == SA_BF16) GO(bf16_t, bf16_t);
     else return SA_ERR_UNSUPPORTED;
 #undef GO
+    SA_LAUNCH_CHECK();
+  }
+  if (num_splits > 1) {
+    hipLaunchKernelGGL(paged_attention_merge_f32_kernel, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml,
+                       (float*)out, D, num_splits);
     SA_LAUNCH_CHECK();
   }
   return 0;

@@ -190,10 +190,12 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Te
 def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                            ctx_len: torch.Tensor, seg_of_token: torch.Tensor, num_tokens: int,
-                           num_heads: int, scale: float, window: Optional[int]) -> torch.Tensor:
+                           num_heads: int, scale: float, window: Optional[int], num_splits: int = 1) -> torch.Tensor:
     """Attention of every token of the step over its request's cached keys (fp32 arithmetic).
 
-    q is the start of the q block of the fused qkv rows (row stride `q_row_stride` elements)."""
+    q is the start of the q block of the fused qkv rows (row stride `q_row_stride` elements).
+    `num_splits` > 1 (float32 only) cuts the keys of every (token, head) into that many parts over
+    the grid, merged by a second kernel: for single tokens over long contexts."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len, seg_of_token)
     P, Hk, page_size, D = k_pages.shape
     _check(v_pages.shape == (P, Hk, D, page_size), "v_pages must be [P, Hk, D, page_size]")
@@ -208,12 +210,19 @@ def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
     _i32(cu_q, B + 1, "cu_q")
     _i32(ctx_len, B, "ctx_len")
     _i32(seg_of_token, T, "seg_of_token")
+    _check(1 <= num_splits <= 64 and (num_splits == 1 or q.dtype == torch.float32),
+           "the keys are cut into 1 to 64 parts, and into more than one in float32 only")
+    part_o = part_ml = None
+    if num_splits > 1:
+        part_o = torch.empty((T * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
     lib = load_library("attention_simple")
     _ret(lib.sa_paged_attention_simple(
         _ptr(q), c_int(q_row_stride), _ptr(out), c_int(_code(q)), _ptr(k_pages), _ptr(v_pages),
         c_int(_code(k_pages)), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len),
         _ptr(seg_of_token), c_int(T), c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size),
-        c_float(scale), c_int(window or 0), _stream()), "paged_attention_simple")
+        c_float(scale), c_int(window or 0), c_int(num_splits), _ptr(part_o), _ptr(part_ml), _stream()),
+        "paged_attention_simple")
     return out
 
 
@@ -266,6 +275,10 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
 # TILED_MIN_CONTEXT on, with the keys cut across workgroups, and the one-wave-per-row kernel below that
 TILED_MIN_ROWS = 16
 TILED_MIN_CONTEXT = 256
+# single tokens of the float32 path whose number times their longest context stays below this take the kernel with a
+# wave per (token, head) and the keys cut into parts; more work takes the tiled kernel (measured at the 1B shape:
+# batch 1 and 8 at contexts around 400 gain 10 and 7 %, batch 8 at 4,096 and batch 64 would lose)
+FP32_ROWWISE_MAX_WORK = 4096
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -652,6 +665,13 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
         if rows > TILED_MIN_ROWS:
             return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                              ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window)
+        if (ctx.max_ctx_len >= TILED_MIN_CONTEXT and q.dtype == torch.float32
+                and ctx.num_tokens * ctx.max_ctx_len <= FP32_ROWWISE_MAX_WORK):
+            # few tokens over not too many keys, a wave per (token, head): parts of 128 keys and more, up to 64
+            splits = max(1, min(64, ctx.max_ctx_len // 128))
+            return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
+                                          ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window,
+                                          splits)
         if ctx.max_ctx_len >= TILED_MIN_CONTEXT:
             # few rows over many keys: about two workgroups per compute unit, parts of at least 256 keys
             tiles = ctx.num_segments * Hk

@@ -262,7 +262,7 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     scale = D ** -0.5
     if kernel == "simple":
         ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
-                                   T, Hq, scale, window)
+                                   T, Hq, scale, window, splits)
     elif kernel == "tiled":
         ops.paged_attention_tiled_f32(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
                                       max(ql for _, ql in segs), Hq, scale, window, splits)
@@ -302,6 +302,18 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
 def test_paged_attention_simple(dtype, Hq, Hk, D, ps):
     segs = [(0, 7), (12, 1), (0, 1), (63, 5), (130, 1), (5, 70)]
     attention_case(dtype, Hq, Hk, D, ps, segs, seed=100 + D)
+
+
+@pytest.mark.parametrize("splits", [2, 5, 64])
+def test_paged_attention_simple_split_keys(splits):
+    """The kernel with a wave per (token, head), float32, keys cut into parts over the grid and merged:
+    more parts than chunks of 64 keys (empty parts), a window, unowned pages NaN."""
+    attention_case("float32", 6, 2, 48, 8, [(700, 1), (0, 1), (63, 1), (300, 1), (129, 1)], seed=500 + splits,
+                   kernel="simple", splits=splits, poison=True)
+    attention_case("float32", 4, 2, 32, 8, [(300, 5), (50, 1), (400, 3)], seed=510 + splits, kernel="simple",
+                   splits=splits, window=100, poison=True)
+    attention_case("float32", 3, 1, 80, 16, [(500, 1), (90, 1)], seed=520 + splits, kernel="simple", splits=splits,
+                   standout=True)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

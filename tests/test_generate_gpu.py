@@ -287,6 +287,84 @@ def test_part_attention_whole_and_in_portions(dtype):
 # ---------------------------------------------------------------------------------------------
 # trace replay as a program
 # ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_part_embedding_and_head(dtype):
+    """The embedding part alone (rows of the table for the step's tokens, fp32 residual stream; a row
+    may take the token that the step before sampled on the device) and the head part alone (fp32
+    logits over a vocabulary that is no power of two, its matrix its own or the table it shares)."""
+    from types import SimpleNamespace
+
+    from serve_amd.parts.standard import LinearHead, TokenEmbedding
+    V, d = 301, 72
+    rt = runtime(dtype)
+    table = rnd((V, d), dtype, 1)
+    emb = TokenEmbedding(vocab_size=V, hidden_size=d)
+    emb.load({"weight": table}, rt)
+    ids = torch.tensor([5, 300, 0, 17], dtype=torch.int32, device=DEV)
+    x = emb.forward(SimpleNamespace(token_ids=ids, src_row=None, prev_tokens=None))
+    assert x.dtype == torch.float32
+    torch.testing.assert_close(x, table[ids.long()].float(), atol=0, rtol=0)
+    # rows 1 and 3 take tokens that were sampled into a device buffer
+    prev = torch.tensor([9, 250, 3], dtype=torch.int32, device=DEV)
+    src = torch.tensor([-1, 2, -1, 0], dtype=torch.int32, device=DEV)
+    x = emb.forward(SimpleNamespace(token_ids=ids, src_row=src, prev_tokens=prev))
+    torch.testing.assert_close(x, table[torch.tensor([5, 3, 0, 9], device=DEV)].float(), atol=0, rtol=0)
+
+    own = rnd((V, d), dtype, 2, 0.1)
+    for tied, tensors, want_w in ((False, {"weight": own}, own), (True, {"weight": table}, table)):
+        head = LinearHead(vocab_size=V, hidden_size=d, tied=tied)
+        req = head.param_requests()[0]
+        assert req.alias_of == "embedding.weight" and req.alias_only == tied
+        head.load(tensors, rt)
+        for rows in (3, 150):
+            h = rnd((rows, d), dtype, 3)
+            logits = head.forward(h)
+            assert logits.dtype == torch.float32 and logits.shape == (rows, V)
+            tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=3e-2, rtol=2e-2)
+            torch.testing.assert_close(logits.double(), h.double() @ want_w.double().T, **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_part_prenorm_residual_arrangement(dtype):
+    """The arrangement alone, around stand-in parts: x + mixer(norm1(x)) is what the second norm sees,
+    the layer hands back the feed-forward's output for the next norm to add, and the stream stays fp32."""
+    from serve_amd.parts.standard import PreNormResidual, RMSNorm
+    d = 64
+    rt = runtime(dtype)
+    seen = {}
+
+    class Mixer:
+        def forward(self, h, ctx, cache, writes_cache=True):
+            seen["mixer_in"] = h.clone()
+            return (h.float() * 2).to(h.dtype)
+
+    class FeedForward:
+        def forward(self, h, ctx):
+            seen["ffn_in"] = h.clone()
+            return (h.float() + 1).to(h.dtype)
+
+    norms = [RMSNorm(size=d, eps=1e-5), RMSNorm(size=d, eps=1e-5)]
+    ws = [rnd((d,), dtype, 1) * 0.1 + 1, rnd((d,), dtype, 2) * 0.1 + 1]
+    for n, w in zip(norms, ws):
+        n.load({"weight": w}, rt)
+    layer = PreNormResidual(mixer=Mixer(), ffn=FeedForward(), mixer_norm=norms[0], ffn_norm=norms[1])
+    assert set(layer.parts()) == set(PreNormResidual.PART_ROLES) and layer.cache_owner() is layer.mixer
+    x = rnd((5, d), torch.float32, 3)
+    pending = rnd((5, d), dtype, 4)
+    x0 = x.clone()
+    out = layer.forward(x, pending, None, None)
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=3e-2, rtol=2e-2)
+    x1 = x0.double() + pending.double()
+    h1 = llama_plain.rms_norm(x1, ws[0].double(), 1e-5)
+    torch.testing.assert_close(seen["mixer_in"].double(), h1, **tol)
+    x2 = x1 + seen["mixer_in"].double() * 2
+    h2 = llama_plain.rms_norm(x2, ws[1].double(), 1e-5)
+    torch.testing.assert_close(seen["ffn_in"].double(), h2, **tol)
+    torch.testing.assert_close(out.double(), seen["ffn_in"].double() + 1, **tol)
+    assert x.dtype == torch.float32
+    torch.testing.assert_close(x.double(), x2, **tol)              # the feed-forward's output is not added yet
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(tmp_path, dtype):
     folder = util.make_folder(tmp_path, "B")

@@ -109,9 +109,11 @@ def decode_run(engine, batch: int, prompt_len: int, warmup: int, steps: int, see
 
 
 def prefill_run(engine, tokens: int, repeats: int, seed: int):
-    """Seconds of one step that runs a whole `tokens`-token prompt (best of `repeats`)."""
+    """Seconds that a whole `tokens`-token prompt takes (best of `repeats`): one step, or with a
+    prompt longer than the engine's portion one step per portion, each over the keys of those before."""
     import torch
     from serve_amd.engine.batch import Segment
+    chunk = min(engine.cfg.prefill_chunk, engine.cfg.max_tokens_per_step)
     best = None
     for i in range(repeats + 1):
         prompt = random_prompts(1, tokens, engine.model.spec.vocab_size, seed + i)[0]
@@ -119,7 +121,9 @@ def prefill_run(engine, tokens: int, repeats: int, seed: int):
         assert engine.runner.admit(rid)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits = engine.runner.step([Segment(rid, prompt, [tokens - 1])])
+        for at in range(0, tokens, chunk):
+            part = prompt[at: at + chunk]
+            logits = engine.runner.step([Segment(rid, part, [len(part) - 1] if at + chunk >= tokens else [])])
         engine.sampler.sample(logits)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
@@ -226,6 +230,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch-1/64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own short JSON line")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="with --prefill-only: the length of the prompt; "
+                    "more than 2,048 tokens are taken in portions of 2,048 (and need --context to hold them)")
     ap.add_argument("--report", action="store_true",
                     help="print a table instead of the JSON line: decode at batch 1, 8 and 64 and the prefill, each "
                     "with its bytes or flops, as a share of the published peaks and of ceilings measured here")
@@ -254,8 +260,11 @@ def main() -> int:
     print(f"[bench] model ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
 
     if args.prefill_only:
-        T = 2048
-        pt = prefill_run(engine, T, repeats=5, seed=7)
+        T = args.prefill_tokens
+        if T < 1 or T > args.context:
+            print("bench.py: --prefill-tokens must lie within --context")
+            return 2
+        pt = prefill_run(engine, T, repeats=5 if T <= 8192 else 2, seed=7)
         print(json.dumps({"prefill": {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
                                       "frac": round(prefill_flops(cfg, T) / pt / peak, 4)}}), flush=True)
         return 0

@@ -492,7 +492,10 @@ __global__ __launch_bounds__(64 * WG_SPLITS) void paged_attention_mfma_wg_kernel
 // Prompt portions (more than 16 rows in a segment).  A workgroup of eight waves takes TW tiles of
 // 32 rows, next to one another in the segment, and walks over the keys in stages of KW * KB blocks
 // of 32 keys (TW * KW = 8).  All eight waves fetch a stage together, 16 bytes a thread at a time,
-// into registers (up to two stages ahead) and from there into LDS one stage ahead; then wave
+// into registers two stages ahead and from there into LDS one stage ahead (K and V^T have two
+// buffers each: while stage i is multiplied from one, stage i + 1 is written to the other, which
+// takes one barrier a stage; a second barrier, with the stage written just before it is read, cost
+// 6 % of the time at head size 64 and 10 % at 128 over long contexts); then wave
 // (tw, kw) multiplies tile tw with the kw-th run of KB blocks of the stage, reading K and V^T from
 // LDS in the lane order of the matrix instruction, with one softmax update (maximum, rescaling of
 // O) for the 32 * KB keys.  The KW waves of a tile hold partial (m, l, O), merged through LDS at
@@ -537,14 +540,12 @@ struct PromptShape {
   static constexpr int K_ROW = HD <= 64 ? 128 : 256;       // bytes of a key's row in LDS
   static constexpr int K_BYTES = KEYS * K_ROW;
   static constexpr int V_BYTES = BLOCKS * HD * 64;
-  static constexpr int STAGE = K_BYTES + V_BYTES;
-  static constexpr int STAGES = 3 * STAGE <= 144 * 1024 ? 3 : 2;
-  static constexpr int LDS_BYTES = STAGES * STAGE;
+  static constexpr int RING_BYTES = 2 * K_BYTES + 2 * V_BYTES;  // two buffers of K, two of V^T
   static constexpr int CHUNKS = 4 * BLOCKS * HD;           // 16-byte pieces of K, and of V, per stage
   static constexpr int PER_THREAD = (CHUNKS + 511) / 512;
-  static constexpr int RING = PER_THREAD <= 2 ? 2 : 1;     // stages held in registers on their way to LDS
   static constexpr int MERGE_FLOATS = DT * 8 + 4;          // per lane: O, m and l of two column tiles
-  static_assert((KW - 1) * TW * MERGE_FLOATS * 64 * 4 <= LDS_BYTES, "the merge reuses the stages' memory");
+  static constexpr int MERGE_BYTES = (KW - 1) * TW * MERGE_FLOATS * 64 * 4;   // the merge reuses the stages' memory
+  static constexpr int LDS_BYTES = RING_BYTES > MERGE_BYTES ? RING_BYTES : MERGE_BYTES;
   static_assert(TW * KW == 8, "eight waves");
 };
 
@@ -616,68 +617,85 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
       v_dim[i] = ch - v_run[i] * HD;
       k_off[i] = v_off[i] = 0;
     }
-    v_lds[i] = S::K_BYTES + ((((v_run[i] >> 2) * HD + v_dim[i]) * 4 + ((v_run[i] & 3) ^ ((v_dim[i] >> 1) & 3))) << 4);
+    v_lds[i] = (((v_run[i] >> 2) * HD + v_dim[i]) * 4 + ((v_run[i] & 3) ^ ((v_dim[i] >> 1) & 3))) << 4;
   }
-  struct Ring {
-    u32x4_t k[PT], v[PT];
+  // page ids of a stage's keys, and of its values, fetched one step before the keys and values are
+  auto lookup_k = [&](int sb, int (&pk)[PT]) __attribute__((always_inline)) {
+    const int key0 = sb * S::KEYS;
+#pragma unroll
+    for (int i = 0; i < PT; ++i)
+      pk[i] = PM == 1 ? bt[min((key0 + k_key[i]) >> page_shift, last_page)] : bt[min((key0 + k_key[i]) / page_size, last_page)];
   };
-  // page ids of a stage, fetched one step before the stage's keys and values are
-  auto lookup = [&](int sb, int (&pk)[PT], int (&pv)[PT * VL]) __attribute__((always_inline)) {
+  auto lookup_v = [&](int sb, int (&pv)[PT * VL]) __attribute__((always_inline)) {
     const int key0 = sb * S::KEYS;
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       if (PM == 1) {
-        pk[i] = bt[min((key0 + k_key[i]) >> page_shift, last_page)];
         pv[i] = bt[min((key0 + v_run[i] * 8) >> page_shift, last_page)];
       } else {
-        pk[i] = bt[min((key0 + k_key[i]) / page_size, last_page)];
 #pragma unroll
         for (int h = 0; h < 2; ++h) pv[i * VL + h] = bt[min((key0 + v_run[i] * 8 + 4 * h) / page_size, last_page)];
       }
     }
   };
   // The loads carry no conditions: a stage beyond the last is read from the last page and never used.
-  auto issue = [&](int sb, const int (&pk)[PT], const int (&pv)[PT * VL], Ring& r) __attribute__((always_inline)) {
+  // With a power-of-two page size, (stage begin mod page) is 0 unless a page holds several stages.
+  auto issue_k = [&](int sb, const int (&pk)[PT], u32x4_t (&r)[PT]) __attribute__((always_inline)) {
     const int key0 = sb * S::KEYS;
     if (PM == 1) {
-      const int in_page = key0 & (page_size - 1);           // 0 unless a page holds several stages
-      const char* kb = k_base + (size_t)in_page * (HD * 2);
-      const char* vb = v_base + (size_t)in_page * 2;
+      const char* kb = k_base + (size_t)(key0 & (page_size - 1)) * (HD * 2);
 #pragma unroll
-      for (int i = 0; i < PT; ++i) {
-        r.k[i] = *reinterpret_cast<const u32x4_t*>(kb + ((uint64_t)(uint32_t)max(pk[i], 0) * page_bytes + (uint32_t)k_off[i]));
-        r.v[i] = *reinterpret_cast<const u32x4_t*>(vb + ((uint64_t)(uint32_t)max(pv[i], 0) * page_bytes + (uint32_t)v_off[i]));
-      }
+      for (int i = 0; i < PT; ++i)
+        r[i] = *reinterpret_cast<const u32x4_t*>(kb + ((uint64_t)(uint32_t)max(pk[i], 0) * page_bytes + (uint32_t)k_off[i]));
     } else {
 #pragma unroll
       for (int i = 0; i < PT; ++i) {
-        const int key = key0 + k_key[i];
-        const int off = key % page_size;
-        r.k[i] = *reinterpret_cast<const u32x4_t*>(k_base + (uint64_t)(uint32_t)max(pk[i], 0) * page_bytes +
-                                                   ((size_t)(hk * page_size + off) * HD + k_seg[i] * 8) * 2);
+        const int off = (key0 + k_key[i]) % page_size;
+        r[i] = *reinterpret_cast<const u32x4_t*>(k_base + (uint64_t)(uint32_t)max(pk[i], 0) * page_bytes +
+                                                 ((size_t)(hk * page_size + off) * HD + k_seg[i] * 8) * 2);
+      }
+    }
+  };
+  auto issue_v = [&](int sb, const int (&pv)[PT * VL], u32x4_t (&r)[PT]) __attribute__((always_inline)) {
+    const int key0 = sb * S::KEYS;
+    if (PM == 1) {
+      const char* vb = v_base + (size_t)(key0 & (page_size - 1)) * 2;
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+        r[i] = *reinterpret_cast<const u32x4_t*>(vb + ((uint64_t)(uint32_t)max(pv[i], 0) * page_bytes + (uint32_t)v_off[i]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const int run = key0 + v_run[i] * 8 + 4 * h;
           const u32x2_t half = *reinterpret_cast<const u32x2_t*>(
               v_base + (uint64_t)(uint32_t)max(pv[i * VL + h], 0) * page_bytes +
               ((size_t)(hk * HD + v_dim[i]) * page_size + run % page_size) * 2);
-          r.v[i][2 * h] = half[0];
-          r.v[i][2 * h + 1] = half[1];
+          r[i][2 * h] = half[0];
+          r[i][2 * h + 1] = half[1];
         }
       }
     }
   };
-  // registers -> LDS.  Values of keys at or beyond the end of the context, and of keys before the
-  // window of the workgroup's first row (their pages may have been given back), hold whatever the
-  // page held before: their probability is 0, and 0 times such a value must stay 0, so they are zeroed.
+  // registers -> LDS: keys into K buffer `buf`, values into V buffer `buf`.  Values of keys at or
+  // beyond the end of the context, and of keys before the window of the workgroup's first row (their
+  // pages may have been given back), hold whatever the page held before: their probability is 0, and
+  // 0 times such a value must stay 0, so they are zeroed.
   int lo_visible = 0;                                       // first key any row of the workgroup's group sees
-  auto stash = [&](int sb, int stage, const Ring& r) __attribute__((always_inline)) {
-    unsigned char* st = smem + stage * S::STAGE;
+  auto stash_k = [&](int buf, const u32x4_t (&r)[PT]) __attribute__((always_inline)) {
+    unsigned char* st = smem + buf * S::K_BYTES;
+#pragma unroll
+    for (int i = 0; i < PT; ++i)
+      if (S::CHUNKS % 512 == 0 || fetches[i]) *reinterpret_cast<u32x4_t*>(st + k_lds[i]) = r[i];
+  };
+  auto stash_v = [&](int sb, int buf, const u32x4_t (&r)[PT]) __attribute__((always_inline)) {
+    unsigned char* st = smem + 2 * S::K_BYTES + buf * S::V_BYTES;
     const int key0 = sb * S::KEYS;
     const bool at_edge = key0 + S::KEYS > ctx || key0 < lo_visible;   // the same for every thread
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
-      u32x4_t v = r.v[i];
+      u32x4_t v = r[i];
       if (at_edge) {
         const int first = key0 + v_run[i] * 8;
 #pragma unroll
@@ -686,10 +704,7 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
           v[e] &= (k0 < ctx && k0 >= lo_visible ? 0x0000ffffu : 0u) | (k1 < ctx && k1 >= lo_visible ? 0xffff0000u : 0u);
         }
       }
-      if (S::CHUNKS % 512 == 0 || fetches[i]) {
-        *reinterpret_cast<u32x4_t*>(st + k_lds[i]) = r.k[i];
-        *reinterpret_cast<u32x4_t*>(st + v_lds[i]) = v;
-      }
+      if (S::CHUNKS % 512 == 0 || fetches[i]) *reinterpret_cast<u32x4_t*>(st + v_lds[i]) = v;
     }
   };
 
@@ -698,7 +713,7 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
   const int kswz = c & 7;                                    // the row's slot mask: (r & 3) | ((r >> 1) & 4), all tiles
   const int ka0 = krow * S::K_ROW + ((g ^ kswz) << 4);       // dims 0..31 (and 64..95, 128 bytes on)
   const int ka1 = krow * S::K_ROW + (((4 + g) ^ kswz) << 4); // dims 32..63 (and 96..127)
-  const int va = S::K_BYTES + (((kw * KB * HD + c) * 4 + (g ^ ((c >> 1) & 3))) << 4);
+  const int va = ((kw * KB * HD + c) * 4 + (g ^ ((c >> 1) & 3))) << 4;
   Frag ones;
   ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);   // bf16 1.0 throughout
 
@@ -759,9 +774,9 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
     struct Scores {
       floatx4_t v[KB][2][NT];
     };
-    // S^T = K Q^T for this wave's KB blocks of LDS stage `stage`
-    auto qk = [&](int stage, Scores& sc) __attribute__((always_inline)) {
-      const unsigned char* st = smem + stage * S::STAGE;
+    // S^T = K Q^T for this wave's KB blocks of the stage in K buffer `buf`
+    auto qk = [&](int buf, Scores& sc) __attribute__((always_inline)) {
+      const unsigned char* st = smem + buf * S::K_BYTES;
       auto& s = sc.v;
 #pragma unroll
       for (int h = 0; h < KB; ++h) {
@@ -787,9 +802,9 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
       }
     };
     // blocks kb .. kb + KB - 1 of the keys: softmax update with their scores, O^T += V^T P^T with
-    // the values of LDS stage `stage`
-    auto softmax_pv = [&](int kb, int stage, Scores& sc) __attribute__((always_inline)) {
-      const unsigned char* st = smem + stage * S::STAGE;
+    // the values in V buffer `buf`
+    auto softmax_pv = [&](int kb, int buf, Scores& sc) __attribute__((always_inline)) {
+      const unsigned char* st = smem + 2 * S::K_BYTES + buf * S::V_BYTES;
       auto& s = sc.v;
       // some key of these blocks is invisible to some row: the causal edge, the window's edge, a
       // block beyond the tile's last key
@@ -880,42 +895,35 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
     };
 
     if (nsb > 0) {
+      // scores, softmax and the product with V of a stage in the same step: in step i, K(i) and V(i)
+      // are read from LDS while K(i + 1) and V(i + 1) are written to the other buffers (one barrier a
+      // step), and stage i + 2 is on its way into registers
       int pk[PT], pv[PT * VL];
-      Ring ra, rb;
-      lookup(s0, pk, pv);
-      issue(s0, pk, pv, ra);
-      lookup(s0 + 1, pk, pv);
-      stash(s0, 0, ra);
-      // one step: stage i + 1 goes from its registers to LDS, the registers are filled again with
-      // the stage RING steps later, then stage i is multiplied
-      int stage = 0;
-      auto step = [&](int i, Ring& r) __attribute__((always_inline)) {
-        const int next = stage + 1 == S::STAGES ? 0 : stage + 1;
-        stash(s0 + i + 1, next, r);
-        issue(s0 + i + 1 + S::RING, pk, pv, r);
-        lookup(s0 + i + 2 + S::RING, pk, pv);
+      u32x4_t rk[PT], rv[PT];
+      lookup_k(s0, pk);
+      lookup_v(s0, pv);
+      issue_k(s0, pk, rk);
+      issue_v(s0, pv, rv);
+      lookup_k(s0 + 1, pk);
+      lookup_v(s0 + 1, pv);
+      stash_k(0, rk);
+      stash_v(s0, 0, rv);
+      issue_k(s0 + 1, pk, rk);
+      issue_v(s0 + 1, pv, rv);
+      lookup_k(s0 + 2, pk);
+      lookup_v(s0 + 2, pv);
+      for (int i = 0; i < nsb; ++i) {
+        const int b = i & 1;
         __syncthreads();
+        stash_k(b ^ 1, rk);
+        stash_v(s0 + i + 1, b ^ 1, rv);
+        issue_k(s0 + i + 2, pk, rk);
+        issue_v(s0 + i + 2, pv, rv);
+        lookup_k(s0 + i + 3, pk);
+        lookup_v(s0 + i + 3, pv);
         Scores sc;
-        qk(stage, sc);
-        softmax_pv(((s0 + i) * KW + kw) * KB, stage, sc);
-        if (S::STAGES == 2) __syncthreads();
-        stage = next;
-      };
-      if (S::RING == 2) {
-        issue(s0 + 1, pk, pv, rb);
-        lookup(s0 + 2, pk, pv);
-        issue(s0 + 2, pk, pv, ra);
-        lookup(s0 + 3, pk, pv);
-        int i = 0;
-        for (; i + 2 <= nsb; i += 2) {
-          step(i, rb);
-          step(i + 1, ra);
-        }
-        if (i < nsb) step(i, rb);
-      } else {
-        issue(s0 + 1, pk, pv, ra);
-        lookup(s0 + 2, pk, pv);
-        for (int i = 0; i < nsb; ++i) step(i, ra);
+        qk(b, sc);
+        softmax_pv(((s0 + i) * KW + kw) * KB, b, sc);
       }
     }
 

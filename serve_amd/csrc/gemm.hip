@@ -73,16 +73,21 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
 }
 
 // The same product for few rows of activations (decode steps of the float32 path), where the work is
-// reading W once: a wave owns RW rows of W, its lanes split K (a float4 each, four per chunk of 1024),
+// reading W once: a wave owns two rows of W, its lanes split K (a float4 each, two per chunk of 512),
 // the MR rows of activations of a pass lie in LDS a chunk at a time, and the lanes' partial sums are
-// added across the wave at the end, always in the same order.  Loads of W carry no conditions: a row
+// added across the wave at the end, always in the same order.  The stream of W never stops: the
+// weights and activations of chunk c + 1 are on their way into registers while chunk c is multiplied
+// (two register sets, two LDS buffers, one barrier a chunk).  Loads of W carry no conditions: a row
 // beyond N is read from the last row and not stored, and beyond K the address wraps to the chunk's
 // begin while the activation operand is zero.  Needs K % 4 == 0 and 16-byte aligned A and W.
-template <int MR, int RW>
+template <int MR>
 __global__ __launch_bounds__(256) void gemm_nt_rows_kernel(const float* __restrict__ A, const float* __restrict__ W,
                                                            float* __restrict__ C, int M, int N, int K) {
-  constexpr int KC = 1024;
-  __shared__ float4 As[MR][KC / 4];
+  constexpr int RW = 2;                               // rows of W per wave (four were no faster, at twice the registers)
+  constexpr int KC = 512;
+  constexpr int NJ = KC / 256;                        // float4 per lane, row of W and chunk
+  constexpr int NA = (MR * (KC / 4) + 255) / 256;     // float4 of activations per thread and chunk
+  __shared__ float4 As[2][MR][KC / 4];
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -96,42 +101,66 @@ __global__ __launch_bounds__(256) void gemm_nt_rows_kernel(const float* __restri
   for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
     for (int r = 0; r < MR; ++r) acc[rw][r] = 0.f;
-  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int k0 = 0; k0 < K; k0 += KC) {
-    __syncthreads();                                  // the chunk before has been used
-    for (int i = tid; i < MR * (KC / 4); i += 256) {
-      const int r = i / (KC / 4);
-      const int c = i - r * (KC / 4);
-      const int k = k0 + c * 4;
-      const int m = m0 + r;
-      As[r][c] = (m < M && k < K) ? *reinterpret_cast<const float4*>(A + (size_t)m * K + k) : zero4;
-    }
-    __syncthreads();
-    float4 w[4][RW];
+  const int nchunks = (K + KC - 1) / KC;
+
+  auto fetch = [&](int c, float4 (&gw)[NJ][RW], float4 (&ga)[NA]) __attribute__((always_inline)) {
+    const int k0 = min(c, nchunks - 1) * KC;          // past the last chunk: read it again, nobody uses it
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const int k = k0 + (j * 64 + lane) * 4;
       const int kc = k < K ? k : k0;                  // beyond K: any valid address, the activations there are 0
 #pragma unroll
-      for (int rw = 0; rw < RW; ++rw) w[j][rw] = *reinterpret_cast<const float4*>(wrow[rw] + kc);
+      for (int rw = 0; rw < RW; ++rw) gw[j][rw] = *reinterpret_cast<const float4*>(wrow[rw] + kc);
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int i = 0; i < NA; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = min(idx / (KC / 4), MR - 1);
+      const int k = k0 + (idx % (KC / 4)) * 4;
+      const int m = m0 + r;
+      ga[i] = *reinterpret_cast<const float4*>(A + (size_t)min(m, M - 1) * K + (k < K ? k : k0));
+    }
+  };
+  auto step = [&](int c, float4 (&cw)[NJ][RW], float4 (&ca)[NA], float4 (&nw)[NJ][RW], float4 (&na)[NA])
+      __attribute__((always_inline)) {
+    const int b = c & 1;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      // (rows beyond M and columns beyond K are zeroed here and not where the loads start: the zeroing waits for them)
+      const int idx = tid + 256 * i;
+      const int r = idx / (KC / 4), col = idx % (KC / 4);
+      const bool inside = m0 + r < M && c * KC + col * 4 < K;
+      float4 v = ca[i];
+      if (!inside) v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (MR * (KC / 4) % 256 == 0 || idx < MR * (KC / 4)) As[b][r][col] = v;
+    }
+    __syncthreads();                                  // (the buffer was last read two chunks ago)
+    fetch(c + 1, nw, na);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
 #pragma unroll
       for (int r = 0; r < MR; ++r) {
-        const float4 a = As[r][j * 64 + lane];
+        const float4 a = As[b][r][j * 64 + lane];
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw) {
           float t = acc[rw][r];
-          t = fmaf(w[j][rw].x, a.x, t);
-          t = fmaf(w[j][rw].y, a.y, t);
-          t = fmaf(w[j][rw].z, a.z, t);
-          t = fmaf(w[j][rw].w, a.w, t);
+          t = fmaf(cw[j][rw].x, a.x, t);
+          t = fmaf(cw[j][rw].y, a.y, t);
+          t = fmaf(cw[j][rw].z, a.z, t);
+          t = fmaf(cw[j][rw].w, a.w, t);
           acc[rw][r] = t;
         }
       }
     }
+  };
+  float4 w0[NJ][RW], w1[NJ][RW], a0[NA], a1[NA];
+  fetch(0, w0, a0);
+  int c = 0;
+  for (; c + 2 <= nchunks; c += 2) {
+    step(c, w0, a0, w1, a1);
+    step(c + 1, w1, a1, w0, a0);
   }
+  if (c < nchunks) step(c, w0, a0, w1, a1);
 #pragma unroll
   for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
@@ -145,15 +174,10 @@ __global__ __launch_bounds__(256) void gemm_nt_rows_kernel(const float* __restri
 
 template <int MR>
 static int launch_rows(const void* A, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
-  // many rows of W: four of them a wave; few: two, so that there are workgroups enough
-  const int rw = N >= 8192 ? 4 : 2;
-  dim3 grid((N + 4 * rw - 1) / (4 * rw), (M + MR - 1) / MR), block(256);
-  if (rw == 4)
-    hipLaunchKernelGGL((gemm_nt_rows_kernel<MR, 4>), grid, block, 0, stream, (const float*)A, (const float*)W,
-                       (float*)C, M, N, K);
-  else
-    hipLaunchKernelGGL((gemm_nt_rows_kernel<MR, 2>), grid, block, 0, stream, (const float*)A, (const float*)W,
-                       (float*)C, M, N, K);
+  // a workgroup of four waves takes eight rows of W
+  dim3 grid((N + 7) / 8, (M + MR - 1) / MR), block(256);
+  hipLaunchKernelGGL((gemm_nt_rows_kernel<MR>), grid, block, 0, stream, (const float*)A, (const float*)W, (float*)C,
+                     M, N, K);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -295,10 +319,13 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
 // are (both measured on an MI355X).  Up to 16 rows always take the first; up to ROWS_KERNEL_MAX_M
 // rows take the one with the smaller estimate (few tiles: a narrow W, decode batches of 17 to 128).
 #define ROWS_KERNEL_MAX_M 128
+#ifndef ROWS_KERNEL_RATE
+#define ROWS_KERNEL_RATE 22e6
+#endif
 static bool rows_kernel_is_faster(int M, int N, int K) {
   if (M <= 16) return true;
   if (M > ROWS_KERNEL_MAX_M) return false;
-  const double rows_us = 2.0 * M * N * K / 22e6;
+  const double rows_us = 2.0 * M * N * K / ROWS_KERNEL_RATE;
   const long long tiles = (long long)((N + 127) / 128) * ((M + 127) / 128);
   const int cus = compute_units();
   const double mfma_us = 0.078 * K * (double)((tiles + cus - 1) / cus);

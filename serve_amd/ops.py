@@ -190,12 +190,11 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Te
 def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                            ctx_len: torch.Tensor, seg_of_token: torch.Tensor, num_tokens: int,
-                           num_heads: int, scale: float, window: Optional[int], num_splits: int = 1) -> torch.Tensor:
-    """Attention of every token of the step over its request's cached keys (fp32 arithmetic).
+                           num_heads: int, scale: float, window: Optional[int]) -> torch.Tensor:
+    """Attention of every token of the step over its request's cached keys (fp32 arithmetic), a wave
+    per (token, head): the general form, for sizes that the other kernels do not take.
 
-    q is the start of the q block of the fused qkv rows (row stride `q_row_stride` elements).
-    `num_splits` > 1 (float32 only) cuts the keys of every (token, head) into that many parts over
-    the grid, merged by a second kernel: for single tokens over long contexts."""
+    q is the start of the q block of the fused qkv rows (row stride `q_row_stride` elements)."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len, seg_of_token)
     P, Hk, page_size, D = k_pages.shape
     _check(v_pages.shape == (P, Hk, D, page_size), "v_pages must be [P, Hk, D, page_size]")
@@ -210,19 +209,12 @@ def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
     _i32(cu_q, B + 1, "cu_q")
     _i32(ctx_len, B, "ctx_len")
     _i32(seg_of_token, T, "seg_of_token")
-    _check(1 <= num_splits <= 64 and (num_splits == 1 or q.dtype == torch.float32),
-           "the keys are cut into 1 to 64 parts, and into more than one in float32 only")
-    part_o = part_ml = None
-    if num_splits > 1:
-        part_o = torch.empty((T * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((T * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
     lib = load_library("attention_simple")
     _ret(lib.sa_paged_attention_simple(
         _ptr(q), c_int(q_row_stride), _ptr(out), c_int(_code(q)), _ptr(k_pages), _ptr(v_pages),
         c_int(_code(k_pages)), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len),
         _ptr(seg_of_token), c_int(T), c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size),
-        c_float(scale), c_int(window or 0), c_int(num_splits), _ptr(part_o), _ptr(part_ml), _stream()),
-        "paged_attention_simple")
+        c_float(scale), c_int(window or 0), _stream()), "paged_attention_simple")
     return out
 
 
@@ -270,15 +262,52 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
     return out
 
 
-# rows (tokens x query heads of a KV head) of the longest segment from which the float32 path's tiled
-# attention is taken whatever the context; with fewer rows (single tokens) it is taken for contexts from
-# TILED_MIN_CONTEXT on, with the keys cut across workgroups, and the one-wave-per-row kernel below that
+def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
+                               v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
+                               ctx_len: torch.Tensor, num_heads: int, scale: float, window: Optional[int],
+                               num_splits: int = 1) -> torch.Tensor:
+    """float32 attention of segments of one token each: a wave takes up to four query heads of a KV
+    head, so that the keys and values are read once for them.  `num_splits` > 1 cuts every key range
+    into that many parts across workgroups, merged by a second kernel."""
+    _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
+    P, Hk, page_size, D = k_pages.shape
+    _check(tiled_attention_available(q, k_pages, q_row_stride),
+           f"paged_attention_decode_f32 takes float32, head sizes 16..128 in steps of 16 and page sizes that are "
+           f"multiples of 4; got head size {D}, page size {page_size}")
+    _check(v_pages.shape == (P, Hk, D, page_size) and v_pages.dtype == torch.float32,
+           "v_pages must be fp32 [P, Hk, D, page_size]")
+    _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
+    _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
+    B = block_table.shape[0]
+    _check(B <= 65535, "paged_attention_decode_f32 takes at most 65,535 segments")
+    _check(out.shape == (B, num_heads * D) and out.dtype == torch.float32,
+           "attention output must be fp32 [B, Hq D]: one token per segment")
+    _check(q.numel() >= (B - 1) * q_row_stride + num_heads * D if B else True, "q is too short")
+    _i32(cu_q, B + 1, "cu_q")
+    _i32(ctx_len, B, "ctx_len")
+    _check(1 <= num_splits <= 64, "num_splits out of range")
+    part_o = part_ml = None
+    if num_splits > 1:
+        part_o = torch.empty((B * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((B * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
+    lib = load_library("attention_simple")
+    _ret(lib.sa_paged_attention_decode_f32(
+        _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(num_heads), c_int(Hk), c_int(D),
+        c_int(page_size), c_float(scale), c_int(window or 0), c_int(num_splits), _ptr(part_o), _ptr(part_ml),
+        _stream()), "paged_attention_decode_f32")
+    return out
+
+
+# The float32 path's attention: steps of single tokens take the kernel with a wave per (segment, up to four
+# heads of a KV head), cut into about FP32_DECODE_WAVES waves along the keys (at the 1B shape, batch 8 and
+# context 4,096: 3.07 ms a step against 4.54 with the tiled kernel, whose workgroups do the arithmetic of 64 rows).
+# Other steps take the tiled kernel when their longest segment has more than TILED_MIN_ROWS rows (tokens x
+# query heads of a KV head) or the context reaches TILED_MIN_CONTEXT (few rows over many keys: the keys cut
+# across workgroups), and the kernel with a wave per (token, head) otherwise.
 TILED_MIN_ROWS = 16
 TILED_MIN_CONTEXT = 256
-# single tokens of the float32 path whose number times their longest context stays below this take the kernel with a
-# wave per (token, head) and the keys cut into parts; more work takes the tiled kernel (measured at the 1B shape:
-# batch 1 and 8 at contexts around 400 gain 10 and 7 %, batch 8 at 4,096 and batch 64 would lose)
-FP32_ROWWISE_MAX_WORK = 4096
+FP32_DECODE_WAVES = 2048
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -603,6 +632,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
         part_o = torch.empty((T * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
     lib = load_library("attention_mfma", {"HEAD_DIM": D})
+    _check(lib.sa_attention_mfma_head_dim() == D, "the attention library was built for another head size")
     _ret(lib.sa_paged_attention_mfma(
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(T), c_int(max_q_len),
@@ -662,16 +692,16 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
     Hk = k_pages.shape[1]
     if tiled_attention_available(q, k_pages, q_row_stride):
         rows = ctx.max_q_len * (num_heads // Hk)
+        if ctx.max_q_len == 1 and ctx.num_tokens == ctx.num_segments <= 65535:
+            # one token a segment: a wave per (segment, up to four heads of a KV head, part of the keys);
+            # about FP32_DECODE_WAVES waves, parts of at least 128 keys
+            waves = ctx.num_segments * Hk * -(-(num_heads // Hk) // 4)
+            splits = max(1, min(64, FP32_DECODE_WAVES // max(waves, 1), ctx.max_ctx_len // 128))
+            return paged_attention_decode_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
+                                              ctx.ctx_len, num_heads, scale, window, splits)
         if rows > TILED_MIN_ROWS:
             return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                              ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window)
-        if (ctx.max_ctx_len >= TILED_MIN_CONTEXT and q.dtype == torch.float32
-                and ctx.num_tokens * ctx.max_ctx_len <= FP32_ROWWISE_MAX_WORK):
-            # few tokens over not too many keys, a wave per (token, head): parts of 128 keys and more, up to 64
-            splits = max(1, min(64, ctx.max_ctx_len // 128))
-            return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
-                                          ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window,
-                                          splits)
         if ctx.max_ctx_len >= TILED_MIN_CONTEXT:
             # few rows over many keys: about two workgroups per compute unit, parts of at least 256 keys
             tiles = ctx.num_segments * Hk

@@ -262,10 +262,13 @@ def attention_case(dtype, Hq, Hk, D, ps, segs, seed, window=None, standout=False
     scale = D ** -0.5
     if kernel == "simple":
         ops.paged_attention_simple(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, seg_of_token,
-                                   T, Hq, scale, window, splits)
+                                   T, Hq, scale, window)
     elif kernel == "tiled":
         ops.paged_attention_tiled_f32(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, T,
                                       max(ql for _, ql in segs), Hq, scale, window, splits)
+    elif kernel == "decode_f32":
+        ops.paged_attention_decode_f32(q, Hq * D, out, k_pages, v_pages, bt.to(DEV), cu_q, ctx_len, Hq, scale,
+                                       window, splits)
     elif kernel == "dispatch":
         # the way the attention part calls it: the step's facts decide how many launches there are
         from types import SimpleNamespace
@@ -304,18 +307,6 @@ def test_paged_attention_simple(dtype, Hq, Hk, D, ps):
     attention_case(dtype, Hq, Hk, D, ps, segs, seed=100 + D)
 
 
-@pytest.mark.parametrize("splits", [2, 5, 64])
-def test_paged_attention_simple_split_keys(splits):
-    """The kernel with a wave per (token, head), float32, keys cut into parts over the grid and merged:
-    more parts than chunks of 64 keys (empty parts), a window, unowned pages NaN."""
-    attention_case("float32", 6, 2, 48, 8, [(700, 1), (0, 1), (63, 1), (300, 1), (129, 1)], seed=500 + splits,
-                   kernel="simple", splits=splits, poison=True)
-    attention_case("float32", 4, 2, 32, 8, [(300, 5), (50, 1), (400, 3)], seed=510 + splits, kernel="simple",
-                   splits=splits, window=100, poison=True)
-    attention_case("float32", 3, 1, 80, 16, [(500, 1), (90, 1)], seed=520 + splits, kernel="simple", splits=splits,
-                   standout=True)
-
-
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_paged_attention_simple_window_and_standout(dtype):
     attention_case(dtype, 4, 2, 32, 8, [(0, 40), (50, 1), (33, 9)], seed=7, window=16)
@@ -351,6 +342,30 @@ def test_paged_attention_tiled_f32_split_keys(splits):
                    standout=True)
     attention_case("float32", 4, 2, 32, 8, [(300, 40), (50, 1), (400, 3)], seed=420 + splits, kernel="tiled",
                    splits=splits, window=100, poison=True)
+
+
+@pytest.mark.parametrize("Hq,Hk,D,ps", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 2, 64, 16), (6, 2, 48, 12), (5, 5, 80, 32),
+                                        (2, 1, 128, 16), (32, 8, 64, 16), (7, 1, 112, 64), (10, 2, 96, 8)])
+@pytest.mark.parametrize("splits", [1, 3, 64])
+def test_paged_attention_decode_f32(Hq, Hk, D, ps, splits):
+    """The float32 path's attention of single tokens (a wave takes up to four query heads of a KV head):
+    groups of one to seven heads, contexts of one key, of less than a block of 64 and of many blocks, whole
+    and cut into parts (more parts than blocks: empty parts); everything unowned holds NaN."""
+    segs = [(700, 1), (0, 1), (63, 1), (64, 1), (1300, 1), (129, 1), (5, 1)]
+    attention_case("float32", Hq, Hk, D, ps, segs, seed=600 + D + splits, kernel="decode_f32", splits=splits,
+                   poison=True)
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+def test_paged_attention_decode_f32_window_and_standout(splits):
+    """A window (the pages before it are given back: -1 in the table, NaN in memory) whose first key lies
+    in the middle of a block of 64 and of a group of four; one far key that dominates."""
+    attention_case("float32", 4, 2, 32, 8, [(300, 1), (50, 1), (401, 1), (99, 1), (100, 1)], seed=620 + splits,
+                   kernel="decode_f32", splits=splits, window=100, poison=True)
+    attention_case("float32", 6, 2, 64, 16, [(1000, 1), (37, 1)], seed=630 + splits, kernel="decode_f32",
+                   splits=splits, window=37, poison=True)
+    attention_case("float32", 3, 1, 80, 16, [(500, 1), (90, 1)], seed=640 + splits, kernel="decode_f32", splits=splits,
+                   standout=True)
 
 
 def test_attention_reduces_to_library_routine():

@@ -5,9 +5,10 @@
 // MFMA kernels do not take.  The reference leaves these products to nn.Linear
 // (serve/model.py:80-82,95,97,159).
 //
-// Three kernels: gemm_nt_rows_kernel for up to 16 rows of float32 activations, gemm_nt_mfma32_kernel
-// (the matrix cores' float32 instruction) for more rows whose length is a multiple of four, and
-// gemm_nt_kernel for everything else: a 256-thread block owns a 64x64 tile of C; K advances in
+// Four kernels: gemm_nt_rows_kernel for up to 16 rows of float32 activations, gemm_nt_mid32_kernel (the
+// matrix cores' float32 instruction, weights streamed once per 64 rows) for 17 to 128,
+// gemm_nt_mfma32_kernel (the same instruction, 128 x 128 tiles) for more rows whose length is a
+// multiple of four, and gemm_nt_kernel for everything else: a 256-thread block owns a 64x64 tile of C; K advances in
 // slices of 16 through LDS; each thread accumulates a 4x4 sub-tile with v_fma_f32.  Every edge (M,
 // N, K not multiples of the tile) is guarded, so any size is accepted.
 #include "common.h"
@@ -183,6 +184,169 @@ static int launch_rows(const void* A, const void* W, void* C, int M, int N, int 
 }
 
 // ---------------------------------------------------------------------------------------------
+// 17 to 128 rows of float32 activations (decode steps of the float32 path at those batch sizes): the
+// weights are streamed once per 64 rows, as in the kernel above, but multiplied on the matrix cores
+// (v_mfma_f32_32x32x2_f32, full float32).  A workgroup of eight waves owns 32 rows of W; the waves
+// are eight slices of each 256-column stage of K (32 columns a wave), their sums are added through
+// LDS at the end, in order.  The MT 32-row tiles of activations of a stage lie in LDS (rows padded
+// by four floats, which spreads the 16-byte reads of the 32 lanes of a column over the banks) and
+// are shared by the eight waves; weights go from global memory straight into registers, two stages
+// ahead of the products, activations one stage ahead.
+// Operands: lane l = (row r = l % 32, half h = l / 32) holds W[n0 + r][k .. k + 3] and
+// A[m0 + r][k .. k + 3] for k = (block of eight columns) + 4 h; component c of both is one
+// instruction's k index h (the order of the columns inside a block of eight does not matter as long
+// as both operands follow it).  Result register e of lane l is C[m0 + l % 32][n0 + 8 (e / 4) + 4 h +
+// e % 4].  Needs K % 4 == 0 and 16-byte aligned A and W; loads carry no conditions (rows beyond M
+// and N are read from the last row, columns beyond K from the stage's begin, with the activation
+// operand zeroed on its way into LDS).
+// ---------------------------------------------------------------------------------------------
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+#define MD_KH 8
+#define MD_KS (32 * MD_KH)                     // columns per stage
+#define MD_PITCH (MD_KS + 4)
+
+template <int MT>
+__global__ __launch_bounds__(64 * MD_KH) void gemm_nt_mid32_kernel(const float* __restrict__ A,
+                                                                   const float* __restrict__ W,
+                                                                   float* __restrict__ C, int M, int N, int K) {
+  constexpr int THREADS = 64 * MD_KH;
+  constexpr int ROWS = 32 * MT;
+  constexpr int NA = ROWS * (MD_KS / 4) / THREADS;            // float4 of activations per thread and stage
+  static_assert(ROWS * (MD_KS / 4) % THREADS == 0, "the activation tile is spread evenly over the threads");
+  static_assert((MD_KH - 1) * MT * 16 * 64 <= ROWS * MD_PITCH, "the sums of the other K slices reuse the tile");
+  __shared__ __attribute__((aligned(16))) float As[ROWS * MD_PITCH];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int kh = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * 32;
+  const int m0 = blockIdx.y * ROWS;
+  const float* wrow = W + (size_t)min(n0 + r, N - 1) * K;
+  // this workgroup's share of the stages of K (gridDim.z parts, each with its own [M, N] of sums)
+  const int all_stages = (K + MD_KS - 1) / MD_KS;
+  const int per_part = (all_stages + gridDim.z - 1) / gridDim.z;
+  const int s_begin = blockIdx.z * per_part;
+  const int nstages = max(0, min(per_part, all_stages - s_begin));
+  C += (size_t)blockIdx.z * M * N;
+
+  floatx16_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[mt][e] = 0.f;
+
+  auto fetch_w = [&](int s, float4 (&w)[4]) __attribute__((always_inline)) {
+    const int k0 = (s_begin + max(0, min(s, nstages - 1))) * MD_KS;   // past the last stage: read it again, nobody uses it
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + kh * 32 + j * 8 + h * 4;
+      w[j] = *reinterpret_cast<const float4*>(wrow + (k < K ? k : k0));
+    }
+  };
+  auto fetch_a = [&](int s, float4 (&a)[NA]) __attribute__((always_inline)) {
+    const int k0 = (s_begin + max(0, min(s, nstages - 1))) * MD_KS;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int idx = tid + THREADS * i;
+      const int row = idx / (MD_KS / 4), col = (idx % (MD_KS / 4)) * 4;
+      a[i] = *reinterpret_cast<const float4*>(A + (size_t)min(m0 + row, M - 1) * K + (k0 + col < K ? k0 + col : k0));
+    }
+  };
+  auto step = [&](int s, float4 (&w)[4], float4 (&wpre)[4], float4 (&a)[NA]) __attribute__((always_inline)) {
+    const int k0 = (s_begin + s) * MD_KS;
+    __syncthreads();                                          // the stage before has been multiplied
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      // (zeroed here and not where the loads start: the zeroing waits for them)
+      const int idx = tid + THREADS * i;
+      const int row = idx / (MD_KS / 4), col = (idx % (MD_KS / 4)) * 4;
+      float4 v = a[i];
+      if (m0 + row >= M || k0 + col >= K) v = make_float4(0.f, 0.f, 0.f, 0.f);
+      *reinterpret_cast<float4*>(&As[row * MD_PITCH + col]) = v;
+    }
+    __syncthreads();
+    fetch_a(s + 1, a);
+    fetch_w(s + 2, wpre);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4 b[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        b[mt] = *reinterpret_cast<const float4*>(&As[(mt * 32 + r) * MD_PITCH + kh * 32 + j * 8 + h * 4]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].x, b[mt].x, acc[mt], 0, 0, 0);
+        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].y, b[mt].y, acc[mt], 0, 0, 0);
+        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].z, b[mt].z, acc[mt], 0, 0, 0);
+        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j].w, b[mt].w, acc[mt], 0, 0, 0);
+      }
+    }
+  };
+
+  float4 w0[4], w1[4], w2[4], a0[NA];
+  fetch_a(0, a0);
+  fetch_w(0, w0);
+  fetch_w(1, w1);
+  // three stages a turn so that the register sets of W take turns without copies
+  int s = 0;
+  for (; s + 3 <= nstages; s += 3) {
+    step(s, w0, w2, a0);
+    step(s + 1, w1, w0, a0);
+    step(s + 2, w2, w1, a0);
+  }
+  if (s < nstages) {
+    step(s, w0, w2, a0);
+    if (s + 1 < nstages) step(s + 1, w1, w0, a0);
+  }
+
+  // add the slices of K in a fixed order: the waves of slices 1.. hand their sums over through LDS
+  __syncthreads();
+  if (kh > 0) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) As[(((kh - 1) * MT + mt) * 16 + e) * 64 + lane] = acc[mt][e];
+  }
+  __syncthreads();
+  if (kh > 0) return;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + mt * 32 + r;
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4) {
+      float v[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int e = e4 * 4 + c;
+        float sum = acc[mt][e];
+#pragma unroll
+        for (int o = 1; o < MD_KH; ++o) sum += As[(((o - 1) * MT + mt) * 16 + e) * 64 + lane];
+        v[c] = sum;
+      }
+      const int n = n0 + e4 * 8 + h * 4;
+      if (m >= M) continue;
+      float* cp = C + (size_t)m * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<float4*>(cp) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (n + c < N) cp[c] = v[c];
+      }
+    }
+  }
+}
+
+template <int MT>
+static int launch_mid32(const void* A, const void* W, void* C, int M, int N, int K, int parts, hipStream_t stream) {
+  dim3 grid((N + 31) / 32, (M + 32 * MT - 1) / (32 * MT), parts), block(64 * MD_KH);
+  hipLaunchKernelGGL((gemm_nt_mid32_kernel<MT>), grid, block, 0, stream, (const float*)A, (const float*)W, (float*)C,
+                     M, N, K);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
 // Many rows (prompt portions of the float32 path, and any mix of storage types): the matrix cores'
 // float32 instruction, v_mfma_f32_32x32x2_f32, which multiplies and adds in full 32-bit precision
 // (it is not the reduced "xf32" mode).  A workgroup of four waves owns a 128 x 128 tile of C, a
@@ -193,7 +357,6 @@ static int launch_rows(const void* A, const void* W, void* C, int M, int N, int 
 // lane l is C[8 (i / 4) + 4 (l / 32) + i % 4][l % 32].  Needs K % 4 == 0 and 16-byte (bf16: 8-byte)
 // aligned rows; rows beyond M and N are read as zeros.
 // ---------------------------------------------------------------------------------------------
-typedef float floatx16_t __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float4 load4f(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ float4 load4f(const bf16_t* p) {
@@ -313,31 +476,41 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
     }
 }
 
-// Which float32 product a shape takes.  gemm_nt_rows_kernel (passes of eight rows, each reading W
-// again) does about 22 TFLOP/s whatever the shape; the matrix-core kernel takes about 0.078 us per
-// element of K for every round of 128 x 128 tiles over the compute units, however few tiles there
-// are (both measured on an MI355X).  Up to 16 rows always take the first; up to ROWS_KERNEL_MAX_M
-// rows take the one with the smaller estimate (few tiles: a narrow W, decode batches of 17 to 128).
-#define ROWS_KERNEL_MAX_M 128
-#ifndef ROWS_KERNEL_RATE
-#define ROWS_KERNEL_RATE 22e6
-#endif
-static bool rows_kernel_is_faster(int M, int N, int K) {
-  if (M <= 16) return true;
-  if (M > ROWS_KERNEL_MAX_M) return false;
-  const double rows_us = 2.0 * M * N * K / ROWS_KERNEL_RATE;
-  const long long tiles = (long long)((N + 127) / 128) * ((M + 127) / 128);
-  const int cus = compute_units();
-  const double mfma_us = 0.078 * K * (double)((tiles + cus - 1) / cus);
-  return rows_us < mfma_us;
+// Which float32 product a shape takes (float32 throughout, K % 4 == 0, 16-byte aligned operands): up
+// to ROWS_KERNEL_MAX_M rows the weight-streaming kernel on the vector ALU (passes of eight rows); from
+// there to MID32_MAX_M rows the matrix-core kernel that streams the weights once per 64 rows (at 64
+// rows and the 1B shape a decode step of the float32 path went from 6.97 to 3.54 ms with it); more
+// rows, and every other mix of types, the tiled kernels below.
+#define ROWS_KERNEL_MAX_M 16
+#define MID32_MAX_M 128
+
+// one or two 32-row tiles of activations a pass (three and four, with the weights read once for up to
+// 128 rows, were no faster at 65 to 96 rows and slower beyond: the matrix cores are the bound there)
+static int pick_mid32(const void* A, const void* W, void* C, int M, int N, int K, int parts, hipStream_t stream) {
+  if (M <= 32) return launch_mid32<1>(A, W, C, M, N, K, parts, stream);
+  return launch_mid32<2>(A, W, C, M, N, K, parts, stream);
+}
+
+// The float32 product of ROWS_KERNEL_MAX_M + 1 to MID32_MAX_M rows with K cut into `parts` (1 to 8) over the
+// grid: C [parts, M, N] takes the partial sums, which the consumer adds in order (narrow matrices have
+// too few rows of W to fill the chip otherwise).  Needs K % 4 == 0 and 16-byte aligned A and W.
+extern "C" int sa_gemm_f32_mid_parts(const void* A, const void* W, void* C, int M, int N, int K, int parts,
+                                     hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K & 3) || parts < 1 || parts > 8 || M <= ROWS_KERNEL_MAX_M || M > MID32_MAX_M ||
+      ((((uintptr_t)A | (uintptr_t)W) & 15) != 0))
+    return SA_ERR_ARG;
+  return pick_mid32(A, W, C, M, N, K, parts, stream);
 }
 
 extern "C" int sa_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                           int M, int N, int K, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return SA_ERR_ARG;
-  if (a_dtype == SA_F32 && w_dtype == SA_F32 && c_dtype == SA_F32 && (K & 3) == 0 && rows_kernel_is_faster(M, N, K) &&
-      (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
+  const bool f32_rows = a_dtype == SA_F32 && w_dtype == SA_F32 && c_dtype == SA_F32 && (K & 3) == 0 &&
+                        (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
+  if (f32_rows && M > ROWS_KERNEL_MAX_M && M <= MID32_MAX_M) return pick_mid32(A, W, C, M, N, K, 1, stream);
+  if (f32_rows && M <= ROWS_KERNEL_MAX_M) {
     if (M == 1) return launch_rows<1>(A, W, C, M, N, K, stream);
     if (M == 2) return launch_rows<2>(A, W, C, M, N, K, stream);
     if (M <= 4) return launch_rows<4>(A, W, C, M, N, K, stream);

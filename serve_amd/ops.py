@@ -155,6 +155,47 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor
     return out
 
 
+# rows of float32 activations that take the matrix-core kernel with the weights streamed once per 64 rows
+F32_MID_MIN_ROWS = 17
+F32_MID_MAX_ROWS = 128
+
+
+def f32_mid_parts(M: int, N: int, K: int) -> int:
+    """Into how many slices the inner dimension of a float32 product of F32_MID_MIN_ROWS..F32_MID_MAX_ROWS
+    rows is cut across workgroups when its consumer adds the parts: a workgroup takes 32 rows of the
+    weights, one per compute unit and pass of 64 rows is wanted, slices of at least 512."""
+    groups = -(-N // 32) * -(-M // 64)
+    cus = compute_units()
+    parts = 1
+    while parts < 8 and groups * parts < cus and K // (parts * 2) >= 512:
+        parts *= 2
+    return parts
+
+
+def gemm_f32_mid_available(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.is_cuda and a.dtype == torch.float32 and w.dtype == torch.float32 and a.dim() == 2 and w.dim() == 2
+            and F32_MID_MIN_ROWS <= a.shape[0] <= F32_MID_MAX_ROWS and a.shape[1] % 4 == 0
+            and a.is_contiguous() and w.is_contiguous() and _aligned16(a, w))
+
+
+def gemm_f32_mid_parts(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[p] = a[:, slice p of K] @ w[:, slice p of K]^T in float32 on the matrix cores, for
+    F32_MID_MIN_ROWS..F32_MID_MAX_ROWS rows: out is fp32 [parts, M, N] (1 to 8 parts), whose sum over the
+    parts is the product; the consumer adds them in order."""
+    _dev(a, w, out)
+    _check(gemm_f32_mid_available(a, w), "gemm_f32_mid_parts takes 17 to 128 rows of contiguous, 16-byte aligned "
+           "float32 with an inner size that is a multiple of 4")
+    M, K = a.shape
+    N = w.shape[0]
+    _check(w.shape[1] == K, f"gemm: inner sizes differ ({K} vs {w.shape[1]})")
+    _check(out.dim() == 3 and out.shape[1:] == (M, N) and 1 <= out.shape[0] <= 8 and out.dtype == torch.float32
+           and out.is_contiguous(), f"gemm_f32_mid_parts: output must be fp32 [1..8, {M}, {N}]")
+    lib = load_library("gemm")
+    _ret(lib.sa_gemm_f32_mid_parts(_ptr(a), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(out.shape[0]),
+                                   _stream()), "gemm_f32_mid_parts")
+    return out
+
+
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
                   slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
                   v_pages: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,

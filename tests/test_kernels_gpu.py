@@ -89,6 +89,23 @@ def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
     torch.testing.assert_close(out.double(), want, **(t32 if c_dt == "float32" else tol("bfloat16")))
 
 
+@pytest.mark.parametrize("M,N,K,parts", [(17, 40, 36, 1), (32, 33, 260, 2), (33, 2048, 2048, 4), (64, 130, 8192, 8),
+                                         (100, 509, 1028, 3), (128, 64, 512, 8), (77, 3072, 516, 1)])
+def test_gemm_f32_mid_parts(M, N, K, parts):
+    """The float32 matrix-core product of 17 to 128 rows with the inner dimension cut into parts over the grid:
+    widths that are no multiple of the 32-row tiles, inner sizes that end in the middle of a stage of 256, more
+    parts than stages (empty parts hold zeros)."""
+    from serve_amd import ops
+    a = rnd((M, K), torch.float32, 14)
+    w = rnd((N, K), torch.float32, 15, 0.1)
+    out = torch.full((parts, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm_f32_mid_parts(a, w, out)
+    want = a.double() @ w.double().T
+    t32 = tol("float32") if K <= 257 else dict(atol=2e-6 * K ** 0.5, rtol=1e-5)
+    torch.testing.assert_close(out.double().sum(0), want, **t32)
+    assert ops.f32_mid_parts(64, 2048, 8192) > 1 and ops.f32_mid_parts(64, 16384, 2048) == 1
+
+
 # ---------------------------------------------------------------------------------------------
 def rope_ref(x, pos, inv_freq, rot, adjacent):
     """x [T, H, D] fp64; complex multiply on the rotated part."""

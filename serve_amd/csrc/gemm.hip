@@ -5,8 +5,8 @@
 // MFMA kernels do not take.  The reference leaves these products to nn.Linear
 // (serve/model.py:80-82,95,97,159).
 //
-// Four kernels: gemm_nt_rows_kernel for up to 16 rows of float32 activations, gemm_nt_mid32_kernel (the
-// matrix cores' float32 instruction, weights streamed once per 64 rows) for 17 to 128,
+// Four kernels: gemm_nt_rows_kernel for up to 8 rows of float32 activations, gemm_nt_mid32_kernel (the
+// matrix cores' float32 instruction, weights streamed once per 64 rows) for 9 to 128,
 // gemm_nt_mfma32_kernel (the same instruction, 128 x 128 tiles) for more rows whose length is a
 // multiple of four, and gemm_nt_kernel for everything else: a 256-thread block owns a 64x64 tile of C; K advances in
 // slices of 16 through LDS; each thread accumulates a 4x4 sub-tile with v_fma_f32.  Every edge (M,
@@ -184,7 +184,7 @@ static int launch_rows(const void* A, const void* W, void* C, int M, int N, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// 17 to 128 rows of float32 activations (decode steps of the float32 path at those batch sizes): the
+// 9 to 128 rows of float32 activations (decode steps of the float32 path at those batch sizes): the
 // weights are streamed once per 64 rows, as in the kernel above, but multiplied on the matrix cores
 // (v_mfma_f32_32x32x2_f32, full float32).  A workgroup of eight waves owns 32 rows of W; the waves
 // are eight slices of each 256-column stage of K (32 columns a wave), their sums are added through
@@ -477,11 +477,12 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma32_kernel(const TA* __restric
 }
 
 // Which float32 product a shape takes (float32 throughout, K % 4 == 0, 16-byte aligned operands): up
-// to ROWS_KERNEL_MAX_M rows the weight-streaming kernel on the vector ALU (passes of eight rows); from
+// to ROWS_KERNEL_MAX_M rows the weight-streaming kernel on the vector ALU; from
 // there to MID32_MAX_M rows the matrix-core kernel that streams the weights once per 64 rows (at 64
-// rows and the 1B shape a decode step of the float32 path went from 6.97 to 3.54 ms with it); more
+// rows and the 1B shape a decode step of the float32 path went from 6.97 to 3.54 ms with it, at 16 rows
+// from 2.89 to 2.58); more
 // rows, and every other mix of types, the tiled kernels below.
-#define ROWS_KERNEL_MAX_M 16
+#define ROWS_KERNEL_MAX_M 8
 #define MID32_MAX_M 128
 
 // one or two 32-row tiles of activations a pass (three and four, with the weights read once for up to

@@ -156,7 +156,7 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor
 
 
 # rows of float32 activations that take the matrix-core kernel with the weights streamed once per 64 rows
-F32_MID_MIN_ROWS = 17
+F32_MID_MIN_ROWS = 9
 F32_MID_MAX_ROWS = 128
 
 
@@ -183,7 +183,7 @@ def gemm_f32_mid_parts(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> t
     F32_MID_MIN_ROWS..F32_MID_MAX_ROWS rows: out is fp32 [parts, M, N] (1 to 8 parts), whose sum over the
     parts is the product; the consumer adds them in order."""
     _dev(a, w, out)
-    _check(gemm_f32_mid_available(a, w), "gemm_f32_mid_parts takes 17 to 128 rows of contiguous, 16-byte aligned "
+    _check(gemm_f32_mid_available(a, w), "gemm_f32_mid_parts takes 9 to 128 rows of contiguous, 16-byte aligned "
            "float32 with an inner size that is a multiple of 4")
     M, K = a.shape
     N = w.shape[0]

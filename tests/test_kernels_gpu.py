@@ -70,11 +70,11 @@ def test_add_rmsnorm(dtype, d, eps):
 @pytest.mark.parametrize("a_dt,w_dt,c_dt", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
                                             ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
 @pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 64, 64), (17, 130, 100), (64, 509, 96), (130, 65, 257),
-                                   # up to 16 rows of float32 with K % 4 == 0: the weight-streaming kernel
+                                   # up to 8 rows of float32 with K % 4 == 0: the weight-streaming kernel; 9 to 128: the
+                                   # matrix cores' float32 instruction with the weights streamed once per 64 rows
                                    (1, 2049, 2048), (8, 509, 1100), (16, 130, 8192), (5, 8200, 36), (2, 3, 4),
                                    (9, 8193, 1028),
-                                   # more rows with K % 4 == 0: the matrix cores' float32 instruction, or (up to
-                                   # 128 rows, where its tiles would be few) the weight-streaming kernel again
+                                   # more rows with K % 4 == 0: the same instruction on 128 x 128 tiles
                                    (200, 300, 2048), (129, 257, 64), (1000, 128, 512), (33, 40, 4), (128, 128, 16),
                                    (100, 2048, 512), (40, 66000, 64)])
 def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
@@ -89,10 +89,10 @@ def test_gemm_nt(a_dt, w_dt, c_dt, M, N, K):
     torch.testing.assert_close(out.double(), want, **(t32 if c_dt == "float32" else tol("bfloat16")))
 
 
-@pytest.mark.parametrize("M,N,K,parts", [(17, 40, 36, 1), (32, 33, 260, 2), (33, 2048, 2048, 4), (64, 130, 8192, 8),
+@pytest.mark.parametrize("M,N,K,parts", [(9, 70, 2048, 2), (17, 40, 36, 1), (32, 33, 260, 2), (33, 2048, 2048, 4), (64, 130, 8192, 8),
                                          (100, 509, 1028, 3), (128, 64, 512, 8), (77, 3072, 516, 1)])
 def test_gemm_f32_mid_parts(M, N, K, parts):
-    """The float32 matrix-core product of 17 to 128 rows with the inner dimension cut into parts over the grid:
+    """The float32 matrix-core product of 9 to 128 rows with the inner dimension cut into parts over the grid:
     widths that are no multiple of the 32-row tiles, inner sizes that end in the middle of a stage of 256, more
     parts than stages (empty parts hold zeros)."""
     from serve_amd import ops

@@ -273,7 +273,9 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
     """float32 attention: 64 rows (tokens x the query heads of a KV head) a workgroup share the keys
     and values of their KV head through LDS (fp32 arithmetic on the vector ALU).  `num_splits` > 1
     cuts the key range of every tile into that many parts across workgroups, merged by a second kernel
-    (for single tokens over long contexts, where there are few tiles)."""
+    (for few rows over long contexts, where there are few tiles; the segments then begin at token 0).
+    The tables may describe a run of the step's segments only: `num_tokens` then counts the tokens up
+    to the end of the last of them, and only their rows of `out` are written."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
     P, Hk, page_size, D = k_pages.shape
     _check(tiled_attention_available(q, k_pages, q_row_stride),
@@ -283,7 +285,8 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
            "v_pages must be fp32 [P, Hk, D, page_size]")
     _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
     T = num_tokens
-    _check(out.shape == (T, num_heads * D) and out.dtype == torch.float32, "attention output must be fp32 [T, Hq D]")
+    _check(out.dim() == 2 and out.shape[0] >= T and out.shape[1] == num_heads * D and out.dtype == torch.float32,
+           "attention output must be fp32 [T, Hq D]")
     _check(q.numel() >= (T - 1) * q_row_stride + num_heads * D if T else True, "q is too short")
     _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
     B = block_table.shape[0]
@@ -307,9 +310,10 @@ def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Te
                                v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                                ctx_len: torch.Tensor, num_heads: int, scale: float, window: Optional[int],
                                num_splits: int = 1) -> torch.Tensor:
-    """float32 attention of segments of one token each: a wave takes up to four query heads of a KV
-    head, so that the keys and values are read once for them.  `num_splits` > 1 cuts every key range
-    into that many parts across workgroups, merged by a second kernel."""
+    """float32 attention of segments of one token each, the step's first B tokens (its tables may be
+    the head of a longer step's): a wave takes up to four query heads of a KV head, so that the keys
+    and values are read once for them.  `num_splits` > 1 cuts every key range into that many parts
+    across workgroups, merged by a second kernel."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
     P, Hk, page_size, D = k_pages.shape
     _check(tiled_attention_available(q, k_pages, q_row_stride),
@@ -321,8 +325,8 @@ def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Te
     _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
     B = block_table.shape[0]
     _check(B <= 65535, "paged_attention_decode_f32 takes at most 65,535 segments")
-    _check(out.shape == (B, num_heads * D) and out.dtype == torch.float32,
-           "attention output must be fp32 [B, Hq D]: one token per segment")
+    _check(out.dim() == 2 and out.shape[0] >= B and out.shape[1] == num_heads * D and out.dtype == torch.float32,
+           "attention output must be fp32 [T, Hq D] with a row for every segment's token")
     _check(q.numel() >= (B - 1) * q_row_stride + num_heads * D if B else True, "q is too short")
     _i32(cu_q, B + 1, "cu_q")
     _i32(ctx_len, B, "ctx_len")
@@ -732,23 +736,30 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
         return out
     Hk = k_pages.shape[1]
     if tiled_attention_available(q, k_pages, q_row_stride):
-        rows = ctx.max_q_len * (num_heads // Hk)
-        if ctx.max_q_len == 1 and ctx.num_tokens == ctx.num_segments <= 65535:
-            # one token a segment: a wave per (segment, up to four heads of a KV head, part of the keys);
-            # about FP32_DECODE_WAVES waves, parts of at least 128 keys
-            waves = ctx.num_segments * Hk * -(-(num_heads // Hk) // 4)
-            splits = max(1, min(64, FP32_DECODE_WAVES // max(waves, 1), ctx.max_ctx_len // 128))
-            return paged_attention_decode_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
-                                              ctx.ctx_len, num_heads, scale, window, splits)
-        if rows > TILED_MIN_ROWS:
-            return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
-                                             ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window)
-        if ctx.max_ctx_len >= TILED_MIN_CONTEXT:
-            # few rows over many keys: about two workgroups per compute unit, parts of at least 256 keys
-            tiles = ctx.num_segments * Hk
-            splits = max(1, min(64, 2 * compute_units() // max(tiles, 1), ctx.max_ctx_len // 256))
-            return paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
-                                             ctx.ctx_len, ctx.num_tokens, ctx.max_q_len, num_heads, scale, window,
-                                             splits)
+        G = num_heads // Hk
+        launches = _attention_launches(ctx)
+        if len(launches) > 1 or ctx.max_q_len == 1 or ctx.max_q_len * G > TILED_MIN_ROWS \
+                or ctx.max_ctx_len >= TILED_MIN_CONTEXT:
+            # decoding requests and prompt portions as two launches, as on the matrix-core path
+            for s0, n, t_end, max_q, max_ctx in launches:
+                whole = s0 == 0 and n == ctx.num_segments
+                bt = block_table if whole else block_table[s0: s0 + n]
+                cu = ctx.cu_q if whole else ctx.cu_q[s0: s0 + n + 1]
+                cl = ctx.ctx_len if whole else ctx.ctx_len[s0: s0 + n]
+                if max_q == 1 and s0 == 0 and n <= 65535:
+                    # one token a segment: a wave per (segment, up to four heads of a KV head, part of the
+                    # keys); about FP32_DECODE_WAVES waves, parts of at least 128 keys
+                    waves = n * Hk * -(-G // 4)
+                    splits = max(1, min(64, FP32_DECODE_WAVES // max(waves, 1), max_ctx // 128))
+                    paged_attention_decode_f32(q, q_row_stride, out, k_pages, v_pages, bt, cu, cl, num_heads, scale,
+                                               window, splits)
+                    continue
+                splits = 1
+                if max_q * G <= TILED_MIN_ROWS and max_ctx >= TILED_MIN_CONTEXT and s0 == 0:
+                    # few rows over many keys: about two workgroups per compute unit, parts of at least 256 keys
+                    splits = max(1, min(64, 2 * compute_units() // max(n * Hk, 1), max_ctx // 256))
+                paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, bt, cu, cl, t_end, max_q,
+                                          num_heads, scale, window, splits)
+            return out
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
                                   ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)

@@ -40,24 +40,23 @@ def model_config(layers: int, shape: str = "llama-1b"):
     return replace(cfg, num_hidden_layers=layers if layers > 0 else cfg.num_hidden_layers)
 
 
-def weight_bytes(cfg, itemsize: int = 2) -> int:
-    d, D = cfg.hidden_size, cfg.head_dim
-    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D * d + d * cfg.num_attention_heads * D
-                 + 3 * d * cfg.intermediate_size + 2 * d)
-    return itemsize * (per_layer * cfg.num_hidden_layers + cfg.vocab_size * d + d)
+def weight_bytes(model, itemsize: int = 2) -> int:
+    """Bytes of weights that a decode step reads: every tensor the model's parts use, once (what each
+    part says of itself, `Part.step_cost`; the rows an embedding gathers are left out)."""
+    elements, _ = model.step_cost(1, logit_rows=1)
+    return itemsize * elements
 
 
-def kv_bytes_per_token(cfg, itemsize: int = 2) -> int:
-    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * itemsize
+def kv_bytes(model, context: float, itemsize: int = 2) -> float:
+    """Bytes of cache that a request with `context` tokens has a decode step read: what every cache
+    layer keeps per token (`Model.cache_elements_per_token`), over the keys it still holds."""
+    return sum(itemsize * n * (context if w is None else min(context, w)) for n, w in model.cache_elements_per_token())
 
 
-def prefill_flops(cfg, T: int) -> float:
-    d, D = cfg.hidden_size, cfg.head_dim
-    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D * d + d * cfg.num_attention_heads * D
-                 + 3 * d * cfg.intermediate_size)
-    matmul = 2.0 * per_layer * cfg.num_hidden_layers * T + 2.0 * cfg.vocab_size * d
-    attention = 4.0 * cfg.num_attention_heads * D * cfg.num_hidden_layers * (T * (T + 1) / 2)
-    return matmul + attention
+def prefill_flops(model, T: int) -> float:
+    """Flops of a whole prompt of T tokens with logits at its last place, by the parts' own accounts."""
+    _, flops = model.step_cost(T, logit_rows=1)
+    return flops
 
 
 def random_prompts(n: int, length: int, vocab: int, seed: int):
@@ -190,7 +189,7 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
 
     def decode_row(eng, batch, prompt_len, w, n):
         dt, mean_ctx = decode_run(eng, batch, prompt_len, w, n, seed=20 + batch)
-        nbytes = weight_bytes(cfg) + batch * mean_ctx * kv_bytes_per_token(cfg)
+        nbytes = weight_bytes(eng.model) + batch * kv_bytes(eng.model, mean_ctx)
         rate = nbytes / (dt / n)
         print(f"{f'decode, batch {batch}, context ~{int(mean_ctx)}':34s} {dt / n * 1e3:8.3f} {batch * n / dt:10.0f} "
               f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}", flush=True)
@@ -199,7 +198,7 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
     decode_row(engine, 8, 4096 - steps - warmup - 3 - head_start(engine, 8, 4096), warmup, steps)
     T = 2048
     pt = prefill_run(engine, T, repeats=5, seed=7)
-    fl = prefill_flops(cfg, T)
+    fl = prefill_flops(engine.model, T)
     print(f"{'prefill, 2,048 tokens':34s} {pt * 1e3:8.3f} {T / pt:10.0f} {fl / 1e12:6.3f} TFLOP {fl / pt / 1e15:7.3f} PFLOP/s "
           f"{fl / pt / BF16_PEAK:8.3f} {fl / pt / ceil['gemm']:11.3f}", flush=True)
     if make_engine is not None:
@@ -266,7 +265,7 @@ def main() -> int:
             return 2
         pt = prefill_run(engine, T, repeats=5 if T <= 8192 else 2, seed=7)
         print(json.dumps({"prefill": {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                                      "frac": round(prefill_flops(cfg, T) / pt / peak, 4)}}), flush=True)
+                                      "frac": round(prefill_flops(engine.model, T) / pt / peak, 4)}}), flush=True)
         return 0
     if args.report:
         def long_engine(batch, context):
@@ -295,7 +294,7 @@ def main() -> int:
     dt, mean_ctx = decode_run(engine, args.batch, prompt_len, warmup, steps, seed=1)
     ms_per_step = dt / steps * 1e3
     value = args.batch * steps / dt
-    step_bytes = weight_bytes(cfg, item) + args.batch * mean_ctx * kv_bytes_per_token(cfg, item)
+    step_bytes = weight_bytes(engine.model, item) + args.batch * kv_bytes(engine.model, mean_ctx, item)
     achieved = step_bytes / (dt / steps)
     rs = cfg.rope_scaling
     rope_text = "none" if rs is None else (f"llama3 factor {rs.factor:g} low {rs.low_freq_factor:g} high "
@@ -319,7 +318,7 @@ def main() -> int:
         T = 2048
         pt = prefill_run(engine, T, repeats=3, seed=7)
         out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                          "frac": round(prefill_flops(cfg, T) / pt / peak, 4)}
+                          "frac": round(prefill_flops(engine.model, T) / pt / peak, 4)}
         points = {}
         for b in (1, 8, 64):
             d, _ = decode_run(engine, b, 256, 4, 250, seed=10 + b)

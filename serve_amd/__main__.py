@@ -44,6 +44,10 @@ def _generate(argv) -> int:
     ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")
     ap.add_argument("--admit-interval", type=int, default=1, help="admit new requests at most every N steps while "
                     "others run, so that the steps between are pure decode steps (1: at every step)")
+    ap.add_argument("--max-graphs", type=int, default=64, help="captured decode steps kept (one per padded batch "
+                    "size and bucket of contexts); the least recently used goes first")
+    ap.add_argument("--debug-poison-cache", action="store_true", help="debugging: cache pages hold NaN until written "
+                    "and again once given back, so that a read of a key that must not be seen shows")
     args = ap.parse_args(argv)
     import torch
 
@@ -52,7 +56,8 @@ def _generate(argv) -> int:
     cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, num_pages=args.num_pages,
                        memory_fraction=args.memory_fraction, max_context=args.max_context,
                        max_requests=args.max_requests, max_tokens_per_step=args.max_tokens_per_step,
-                       prefill_chunk=args.prefill_chunk, admission=args.admission, admit_interval=args.admit_interval, seed=args.seed)
+                       prefill_chunk=args.prefill_chunk, admission=args.admission, admit_interval=args.admit_interval, seed=args.seed,
+                       max_graphs=args.max_graphs, debug_poison_cache=args.debug_poison_cache)
     if args.model:
         engine = Engine.from_folder(args.model, cfg)
     else:

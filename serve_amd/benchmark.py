@@ -98,6 +98,9 @@ def main(argv=None) -> int:
                          "(serve/run.py:265) beside decode steps of their own")
     ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")
+    ap.add_argument("--phases", action="store_true", help="time the host's phases of the timed run (schedule, "
+                    "plan_step, stage_copy, launch, read_back, ...) with named ranges and print their totals; the "
+                    "ranges are also roctx markers for `rocprofv3 --marker-trace`")
     ap.add_argument("--admit-interval", type=int, default=1, help="admit new requests at most every N steps while "
                     "others run, so that the steps between are pure decode steps (1: at every step)")
     args = ap.parse_args(argv)
@@ -108,12 +111,12 @@ def main(argv=None) -> int:
                        max_tokens_per_step=args.max_tokens_per_step or 2048 + args.max_requests,
                        prefill_chunk=args.prefill_chunk,
                        admission=args.admission, admit_interval=args.admit_interval, seed=args.seed)
-    print(f"loading model {args.model or args.shape}...")
+    print(f"loading {args.model or args.shape} ({args.dtype}) ...", flush=True)
     if args.model:
         engine = Engine.from_folder(args.model, cfg)
     else:
         engine = Engine.from_config(SHAPES[args.shape], args.seed, cfg)
-    print(f"Model finished loading; cache of {engine.runner.num_pages} pages of {args.page_size} tokens")
+    print(f"model on the device; cache: {engine.runner.num_pages} pages of {args.page_size} tokens per group")
     requests = generate_requests(args.input_length, args.output_length, args.num_sequences,
                                  engine.model.spec.vocab_size, args.fixed_lengths,
                                  min_input_length=args.min_input_length, fixed_output_length=args.fixed_output_length)
@@ -121,35 +124,48 @@ def main(argv=None) -> int:
     def fn():
         return engine.generate(requests, args.temperature)
 
-    print("doing first run")
+    print(f"first run of {len(requests)} requests (loads the kernels, captures the graphs) ...", flush=True)
     st = time.perf_counter()
     fn()
     torch.cuda.synchronize()
-    print(f"Warmup time: {time.perf_counter() - st:.4f} seconds")
+    print(f"first run: {time.perf_counter() - st:.4f} s")
     if not args.profile_only:
+        from . import trace
+        if args.phases:
+            trace.enable()
+            trace.reset()
         torch.cuda.synchronize()
         st = time.perf_counter()
         responses = fn()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - st
+        if args.phases:
+            trace.disable()
         total = sum(len(r.generated_tokens) for r in responses)
         failed = [(i, r.error) for i, r in enumerate(responses) if r.error]
         if failed:
             print(f"{len(failed)} requests did not run; the first: request {failed[0][0]}: {failed[0][1]}",
                   file=sys.stderr)
             return 1
-        print(f"Time taken: {elapsed:.4f} seconds")
-        print(f"Throughput: {total / elapsed:.2f} tokens/second")
+        print(f"timed run: {elapsed:.4f} s for {total} generated tokens")
+        print(f"generated tokens per second: {total / elapsed:.2f}")
+        if args.phases:
+            print("host time inside the named ranges of the timed run (ranges nest: launch holds write_to_cache "
+                  "and attention):")
+            print(trace.report(elapsed))
     if args.profile or args.profile_only:
         import os
         name = f"generate_{args.input_length}_{args.output_length}_{args.num_sequences}"
+        from . import trace
+        trace.enable(markers=False, torch_ranges=True)
         with torch.profiler.profile() as prof:
             with torch.autograd.profiler.record_function(name):
                 fn()
+        trace.disable()
         os.makedirs("/tmp/traces", exist_ok=True)
         path = f"/tmp/traces/trace_{name}_{time.strftime('%H%M')}.json"
         prof.export_chrome_trace(path)
-        print(f"Trace saved to {path}")
+        print(f"profiler trace written to {path}")
     return 0
 
 

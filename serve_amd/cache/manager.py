@@ -91,6 +91,9 @@ class CacheManager:
         # the block tables once more as one int32 matrix per group, row = state slot, so that a
         # step can gather the rows of its requests without walking Python lists
         self.table_rows = [np.zeros((max_requests, max_pages_per_request), dtype=np.int32) for _ in windows]
+        # called with (group, page ids) whenever pages return to a pool (a debugging hook: the owner of
+        # the device memory may overwrite what they held)
+        self.on_free = None
 
     # -- queries --------------------------------------------------------------------------------
     @property
@@ -120,6 +123,22 @@ class CacheManager:
 
     def pages_for_tokens(self, n_tokens: int) -> int:
         return -(-n_tokens // self.page_size)
+
+    def max_pages_for(self, n_tokens: int, portion: int = 1) -> List[int]:
+        """Per group: the most pages a request holds at any time on its way to `n_tokens` tokens
+        when it is fed in portions of at most `portion` tokens and trimmed after every step.  A
+        group that keeps every key needs the pages of all its tokens; a group that keeps a window
+        of W keys never holds more than the window, one portion and the page their first key
+        shares with keys that have gone."""
+        ps = self.page_size
+        whole = -(-n_tokens // ps)
+        out = []
+        for w in self.windows:
+            if w is None:
+                out.append(whole)
+            else:
+                out.append(min(whole, -(-(w - 1 + max(1, portion)) // ps) + 1))
+        return out
 
     def _first_live_index(self, group: int, n_tokens: int) -> int:
         """Index of the first page a query at position >= n_tokens can still see."""
@@ -188,6 +207,8 @@ class CacheManager:
             gone = [p for p in table[:first] if p != FREED]
             if gone:
                 self.pools[g].give_back(gone)
+                if self.on_free is not None:
+                    self.on_free(g, gone)
                 for i in range(first):
                     table[i] = FREED
                 self.table_rows[g][r.slot, :first] = FREED
@@ -200,7 +221,10 @@ class CacheManager:
         if r is None:
             raise CacheError(f"request {req_id!r} is released but not admitted")
         for g, table in enumerate(r.tables):
-            self.pools[g].give_back([p for p in table if p != FREED])
+            held = [p for p in table if p != FREED]
+            self.pools[g].give_back(held)
+            if self.on_free is not None and held:
+                self.on_free(g, held)
             self.table_rows[g][r.slot, : len(table)] = 0
         self._free_slots.append(r.slot)
 

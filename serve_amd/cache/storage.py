@@ -45,7 +45,11 @@ def bytes_per_page(requests: Sequence[Optional[TokenCacheRequest]], windows: Seq
 class CacheStorage:
     def __init__(self, rt: Runtime, cache_requests: Sequence[Optional[TokenCacheRequest]],
                  state_requests: Sequence[Optional[StateRequest]], windows: Sequence[Optional[int]],
-                 num_pages: Sequence[int], page_size: int, max_requests: int):
+                 num_pages: Sequence[int], page_size: int, max_requests: int, poison: bool = False):
+        """`poison` (debugging): pages hold NaN until a token is stored in them, and again once they
+        are given back (`poison_pages`): a kernel that reads a key it must not see then shows in the
+        logits."""
+        self.poison = bool(poison)
         self.layers: List[LayerCache] = []
         for cr, sr in zip(cache_requests, state_requests):
             lc = LayerCache(page_size=page_size)
@@ -60,6 +64,8 @@ class CacheStorage:
                     # would carry into a masked position's product
                     lc.pages[t.name] = torch.zeros((num_pages[g],) + t.page_shape(page_size),
                                                    dtype=t.dtype or rt.dtype, device=rt.device)
+                    if self.poison and lc.pages[t.name].is_floating_point():
+                        lc.pages[t.name].fill_(float("nan"))
             if sr is not None:
                 lc.state = torch.zeros((max_requests,) + tuple(sr.shape), dtype=sr.dtype, device=rt.device)
             self.layers.append(lc)
@@ -68,3 +74,16 @@ class CacheStorage:
         for lc in self.layers:
             if lc.state is not None:
                 lc.state[slot].zero_()
+
+    def poison_pages(self, group: int, pages: Sequence[int]) -> None:
+        """Overwrite the given pages of every layer of the group with NaN (pages that went back to
+        the pool, in the debugging mode)."""
+        if not pages:
+            return
+        for lc in self.layers:
+            if lc.group != group:
+                continue
+            idx = torch.as_tensor(list(pages), dtype=torch.long, device=next(iter(lc.pages.values())).device)
+            for t in lc.pages.values():
+                if t.is_floating_point():
+                    t[idx] = float("nan")

@@ -35,9 +35,16 @@ class EngineConfig:
     device: str = "cuda:0"
     # replay a decode-only step from a captured HIP graph
     use_graphs: bool = True
+    # how many captured steps (one per padded batch size and bucket of contexts) are kept; beyond
+    # that the least recently used one is dropped and captured again when its shape comes back
+    max_graphs: int = 64
     # launch a decode step before the previous step's tokens have reached the host (they are fed
     # back on the device); needs graphs, no stop tokens and nobody keeping logits
     async_decode: bool = True
+
+    # debugging: every page of the cache holds NaN until a token is stored in it and again once it is
+    # given back, so that a kernel reading a key it must not see shows in the logits
+    debug_poison_cache: bool = False
 
     def validate(self) -> None:
         if self.dtype not in DTYPES:
@@ -52,6 +59,8 @@ class EngineConfig:
             raise ValueError("prefill_chunk must be positive")
         if self.admit_interval < 1:
             raise ValueError("admit_interval must be at least 1")
+        if self.max_graphs < 1:
+            raise ValueError("max_graphs must be at least 1")
 
     @property
     def max_pages_per_request(self) -> int:

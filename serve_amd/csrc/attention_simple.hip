@@ -549,16 +549,19 @@ static int launch_decode_f32(const void* q, int q_stride, void* out, const void*
 
 // float32 attention of B segments of one token each (token r is the last of a context of ctx_len[r]
 // tokens) over their cached keys.  D a multiple of 16 up to 128, page_size a multiple of 4.
-// num_splits > 1 cuts every key range into that many parts over the grid; part_o [B Hq num_splits, D]
-// and part_ml [B Hq num_splits, 2] (fp32) then take the parts, which a second kernel merges.
+// The segments are a run of the step's tokens: segment i is token first_token + i (cu_q[i] must say
+// so; the host knows it and the kernels do not check it), which is the row of q, out and the parts it
+// uses.  num_splits > 1 cuts every key range into that many parts over the grid; part_o
+// [(first_token + B) Hq num_splits, D] and part_ml [(first_token + B) Hq num_splits, 2] (fp32) then
+// take the parts, which a second kernel merges for the rows first_token .. first_token + B - 1.
 extern "C" int sa_paged_attention_decode_f32(const void* q, int q_stride, void* out, const void* k_pages,
                                              const void* v_pages, const int* block_table, int max_pages,
-                                             const int* cu_q, const int* ctx_len, int B, int Hq, int Hk, int D,
-                                             int page_size, float scale, int window, int num_splits, float* part_o,
-                                             float* part_ml, hipStream_t stream) {
+                                             const int* cu_q, const int* ctx_len, int B, int first_token, int Hq,
+                                             int Hk, int D, int page_size, float scale, int window, int num_splits,
+                                             float* part_o, float* part_ml, hipStream_t stream) {
   if (B <= 0) return 0;
   if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > 128 || (D & 15) || page_size <= 0 || (page_size & 3) ||
-      max_pages <= 0 || (q_stride & 3) || num_splits < 1 || num_splits > 64)
+      max_pages <= 0 || (q_stride & 3) || num_splits < 1 || num_splits > 64 || first_token < 0)
     return SA_ERR_ARG;
   if (num_splits > 1 && (!part_o || !part_ml)) return SA_ERR_ARG;
   int rc = SA_ERR_ARG;
@@ -579,8 +582,10 @@ extern "C" int sa_paged_attention_decode_f32(const void* q, int q_stride, void* 
   }
 #undef GO
   if (rc != 0 || num_splits == 1) return rc;
-  hipLaunchKernelGGL(paged_attention_merge_f32_kernel, dim3((unsigned)B * Hq), dim3(64), 0, stream, part_o, part_ml,
-                     (float*)out, D, num_splits);
+  const size_t row0 = (size_t)first_token * Hq;
+  hipLaunchKernelGGL(paged_attention_merge_f32_kernel, dim3((unsigned)B * Hq), dim3(64), 0, stream,
+                     part_o + row0 * num_splits * D, part_ml + row0 * num_splits * 2, (float*)out + row0 * D, D,
+                     num_splits);
   SA_LAUNCH_CHECK();
   return 0;
 }

@@ -4,7 +4,8 @@
 // is launched kernel by kernel calls this a hundred times, so what a call costs on the host counts:
 // the descriptors and the algorithm of a shape are looked up once and kept (a plan per device, M, N,
 // K and output type), and a call is one hipblasLtMatmul with them.  Nothing is allocated here: the
-// caller brings the workspace.
+// caller brings the workspace.  The library handle of a device and the plans live until the process
+// ends.
 //
 // Row-major C = A W^T is, in the column-major terms of the library, C^T[N, M] = op_T(W) A^T with W
 // seen as a K x N matrix of leading dimension K and A as a K x M matrix of leading dimension K.
@@ -23,6 +24,7 @@ struct Plan {
   hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
+  int failed = 0;            // the error of a shape that could not be planned (then nothing else is set)
 };
 
 constexpr int MAX_DEVICES = 64;
@@ -36,8 +38,16 @@ std::map<std::tuple<int, int, int, int, int, size_t>, Plan> plans;   // (device,
     if (st__ != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)st__; \
   } while (0)
 
-// the plan of a shape, made at its first call (the lock is held)
-int make_plan(hipblasLtHandle_t handle, int M, int N, int K, int c_dtype, size_t workspace_bytes, Plan* plan) {
+void destroy_plan(Plan* plan) {
+  if (plan->desc) hipblasLtMatmulDescDestroy(plan->desc);
+  if (plan->w) hipblasLtMatrixLayoutDestroy(plan->w);
+  if (plan->a) hipblasLtMatrixLayoutDestroy(plan->a);
+  if (plan->c) hipblasLtMatrixLayoutDestroy(plan->c);
+  plan->desc = nullptr;
+  plan->w = plan->a = plan->c = nullptr;
+}
+
+int fill_plan(hipblasLtHandle_t handle, int M, int N, int K, int c_dtype, size_t workspace_bytes, Plan* plan) {
   const hipDataType out = c_dtype == SA_F32 ? HIP_R_32F : HIP_R_16BF;
   LT_CHECK(hipblasLtMatmulDescCreate(&plan->desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   const int32_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
@@ -64,6 +74,16 @@ int make_plan(hipblasLtHandle_t handle, int M, int N, int K, int c_dtype, size_t
   return 0;
 }
 
+// the plan of a shape, made at its first call (the lock is held).  A shape that cannot be planned
+// keeps its error code (`failed`) and nothing else, so that it is neither planned again at every
+// call nor leaves descriptors behind.
+int make_plan(hipblasLtHandle_t handle, int M, int N, int K, int c_dtype, size_t workspace_bytes, Plan* plan) {
+  const int rc = fill_plan(handle, M, N, K, c_dtype, workspace_bytes, plan);
+  if (rc != 0) destroy_plan(plan);
+  plan->failed = rc;
+  return rc;
+}
+
 }  // namespace
 
 // C = A W^T through hipBLASLt.  c_dtype SA_BF16 or SA_F32; `workspace` of `workspace_bytes` bytes is
@@ -85,11 +105,11 @@ extern "C" int sa_blaslt_mm(const void* A, const void* W, void* C, int c_dtype, 
     auto it = plans.find(key);
     if (it == plans.end()) {
       Plan fresh;
-      const int rc = make_plan(handle, M, N, K, c_dtype, workspace_bytes, &fresh);
-      if (rc != 0) return rc;
+      make_plan(handle, M, N, K, c_dtype, workspace_bytes, &fresh);
       it = plans.emplace(key, fresh).first;
     }
     plan = &it->second;                      // (entries of a std::map stay where they are)
+    if (plan->failed != 0) return plan->failed;
   }
   if (plan->workspace > workspace_bytes) return SA_ERR_ARG;
   const float one = 1.f, zero = 0.f;

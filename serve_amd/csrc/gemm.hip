@@ -223,10 +223,10 @@ __global__ __launch_bounds__(64 * MD_KH) void gemm_nt_mid32_kernel(const float* 
   const int m0 = blockIdx.y * ROWS;
   const float* wrow = W + (size_t)min(n0 + r, N - 1) * K;
   // this workgroup's share of the stages of K (gridDim.z parts, each with its own [M, N] of sums)
+  // (spread evenly: no part is empty while there are at least as many stages as parts)
   const int all_stages = (K + MD_KS - 1) / MD_KS;
-  const int per_part = (all_stages + gridDim.z - 1) / gridDim.z;
-  const int s_begin = blockIdx.z * per_part;
-  const int nstages = max(0, min(per_part, all_stages - s_begin));
+  const int s_begin = (int)((long long)blockIdx.z * all_stages / gridDim.z);
+  const int nstages = (int)((long long)(blockIdx.z + 1) * all_stages / gridDim.z) - s_begin;
   C += (size_t)blockIdx.z * M * N;
 
   floatx16_t acc[MT];
@@ -236,7 +236,8 @@ __global__ __launch_bounds__(64 * MD_KH) void gemm_nt_mid32_kernel(const float* 
     for (int e = 0; e < 16; ++e) acc[mt][e] = 0.f;
 
   auto fetch_w = [&](int s, float4 (&w)[4]) __attribute__((always_inline)) {
-    const int k0 = (s_begin + max(0, min(s, nstages - 1))) * MD_KS;   // past the last stage: read it again, nobody uses it
+    // past the part's last stage: read it again, nobody uses it (a part without stages reads the matrix's last one)
+    const int k0 = min(s_begin + max(0, min(s, nstages - 1)), all_stages - 1) * MD_KS;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = k0 + kh * 32 + j * 8 + h * 4;
@@ -244,7 +245,7 @@ __global__ __launch_bounds__(64 * MD_KH) void gemm_nt_mid32_kernel(const float* 
     }
   };
   auto fetch_a = [&](int s, float4 (&a)[NA]) __attribute__((always_inline)) {
-    const int k0 = (s_begin + max(0, min(s, nstages - 1))) * MD_KS;
+    const int k0 = min(s_begin + max(0, min(s, nstages - 1)), all_stages - 1) * MD_KS;
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       const int idx = tid + THREADS * i;
@@ -287,17 +288,36 @@ __global__ __launch_bounds__(64 * MD_KH) void gemm_nt_mid32_kernel(const float* 
   fetch_a(0, a0);
   fetch_w(0, w0);
   fetch_w(1, w1);
-  // three stages a turn so that the register sets of W take turns without copies
-  int s = 0;
+  // three stages a turn so that the register sets of W take turns without copies.  Sums in two
+  // levels, as in the kernel for many rows below: an accumulator takes the 480 terms of five turns and
+  // is then added to the wave's total, so that a long inner dimension does not round 1,800 terms
+  // into one running sum.
+  floatx16_t total[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) total[mt][e] = 0.f;
+  int s = 0, turns = 0;
   for (; s + 3 <= nstages; s += 3) {
     step(s, w0, w2, a0);
     step(s + 1, w1, w0, a0);
     step(s + 2, w2, w1, a0);
+    if (++turns == 5) {
+      turns = 0;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        total[mt] += acc[mt];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[mt][e] = 0.f;
+      }
+    }
   }
   if (s < nstages) {
     step(s, w0, w2, a0);
     if (s + 1 < nstages) step(s + 1, w1, w0, a0);
   }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] += total[mt];
 
   // add the slices of K in a fixed order: the waves of slices 1.. hand their sums over through LDS
   __syncthreads();

@@ -527,18 +527,9 @@ static bool takes_skinny(int M, int N, const QkvRopeArgs& qa) {
 }
 
 // workgroup shapes (row groups x K slices) of products with 65 to 128 rows of activations
-#ifndef MID8_PLAIN_NR
-#define MID8_PLAIN_NR 2
-#define MID8_PLAIN_KH 4
-#endif
-#ifndef MID8_SWIGLU_NR
-#define MID8_SWIGLU_NR 2
-#define MID8_SWIGLU_KH 4
-#endif
-#ifndef MID8_HEAD_NR
-#define MID8_HEAD_NR 4
-#define MID8_HEAD_KH 2
-#endif
+constexpr int MID8_PLAIN_NR = 2, MID8_PLAIN_KH = 4;
+constexpr int MID8_SWIGLU_NR = 2, MID8_SWIGLU_KH = 4;
+constexpr int MID8_HEAD_NR = 4, MID8_HEAD_KH = 2;
 
 template <typename TC, int EPI>
 static int pick_mid(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,

@@ -15,8 +15,8 @@ int sa_sample(const float* logits, const float* temperature, const unsigned long
               float* part_v, int* part_i, int R, int V, hipStream_t stream);
 
 // sa_sample for callers that cannot allocate device memory (code under HIP graph capture, tight
-// serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
-// sampling allocates through torch (serve/run.py:48-60).  The same kernels as sa_sample; the
+// serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+// The same kernels as sa_sample; the
 // per-chunk partial results lie in an array that the library holds on every GPU it runs on
 // (SA_SAMPLE_NOALLOC_ENTRIES entries of 8 bytes, 512 KiB, kept until the process ends) instead of
 // in arrays the caller brings.  The call allocates nothing and frees nothing.

@@ -62,6 +62,8 @@ class StepContext:
     # decode steps replayed from a graph: rows whose token comes from the device (see runner)
     src_row: Optional[torch.Tensor] = None
     prev_tokens: Optional[torch.Tensor] = None
+    # where the head is asked to put the step's logits (fp32 [R, V]); None: wherever it likes
+    logits_out: Optional[torch.Tensor] = None
 
 
 def _align(n: int) -> int:

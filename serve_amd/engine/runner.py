@@ -7,19 +7,20 @@ decoded tokens together, cut anywhere, and runs only the tokens it is given.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
 
-from .. import ops
+from .. import ops, trace
 
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage, bytes_per_page, group_windows
 from ..config.engine import EngineConfig
 from ..models.model import Model
 from ..parts.base import Runtime
-from .batch import Segment, StepLayout, build_step, context_from, plan_step
+from .batch import Segment, StepLayout, context_from, plan_step
 
 # padded batch sizes for which decode-only steps are captured into graphs
 GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
@@ -45,7 +46,7 @@ class _GraphEntry:
         self.host_tokens = [torch.zeros(b_pad, dtype=torch.int32).pin_memory() for _ in range(2)]
         self.copied = torch.cuda.Event()
         self.graph = None
-        self.logits = None
+        self.keeps_logits = False          # whether the captured step leaves its logits in the runner's buffer
         self.runs = 0
         self.launches = 0
 
@@ -61,8 +62,9 @@ class DecodeHandle:
         self.host_tokens, self.event, self.n = host_tokens, event, n
 
     def tokens(self) -> List[int]:
-        self.event.synchronize()
-        return self.host_tokens[: self.n].tolist()
+        with trace.span("read_back"):
+            self.event.synchronize()
+            return self.host_tokens[: self.n].tolist()
 
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -101,9 +103,17 @@ class ModelRunner:
         self.num_pages = num_pages
         self.cache = CacheManager(self.windows, num_pages, cfg.page_size, cfg.max_requests,
                                   cfg.max_pages_per_request)
-        self.storage = CacheStorage(rt, creq, sreq, self.windows, num_pages, cfg.page_size, cfg.max_requests)
-        self._graphs = {}
+        self.storage = CacheStorage(rt, creq, sreq, self.windows, num_pages, cfg.page_size, cfg.max_requests,
+                                    poison=cfg.debug_poison_cache)
+        if cfg.debug_poison_cache:
+            self.cache.on_free = self.storage.poison_pages
+        # captured decode steps by (padded batch, bucket of contexts), least recently used first; at most
+        # cfg.max_graphs of them are kept
+        self._graphs = OrderedDict()
         self._graph_pool = None
+        # the fp32 logits of every graph-replayed step: one buffer for all graphs (they never run side
+        # by side), made at the first such step
+        self._graph_logits = None
         # tokens sampled by the latest decode launch, by row: the next launch may read them here
         self.sampled = torch.zeros(max(ASYNC_GRAPH_BATCHES[-1], cfg.max_requests), dtype=torch.int32, device=rt.device)
         self._row_of = {}
@@ -122,7 +132,8 @@ class ModelRunner:
         return True
 
     def release(self, req_id) -> None:
-        self.cache.release(req_id)
+        with trace.span("free_request"):
+            self.cache.release(req_id)
 
     def forget_launches(self) -> None:
         """Drop what is remembered of steps launched ahead of the host (after a failed run)."""
@@ -143,8 +154,12 @@ class ModelRunner:
                 if not borrow:
                     logits = logits.clone()
             else:
-                ctx = build_step(segments, self.cache, self.vocab_size, self.rt.device)
-                logits = self.model.forward(ctx, self.storage.layers)
+                with trace.span("plan_step"):
+                    lay, host, facts = plan_step(segments, self.cache, self.vocab_size)
+                with trace.span("stage_copy"):
+                    ctx = context_from(lay, torch.from_numpy(host).to(self.rt.device), facts)
+                with trace.span("launch"):
+                    logits = self.model.forward(ctx, self.storage.layers)
                 ctx_lens = ctx.ctx_lens
         for s, n in zip(segments, ctx_lens):
             self.cache.trim(s.req_id, n)
@@ -170,62 +185,86 @@ class ModelRunner:
             bucket *= 2
         # the block tables of a shape are as wide as its bucket of contexts needs, no wider
         mp = min(self.cfg.max_pages_per_request, -(-bucket // self.cfg.page_size))
-        lay, host, facts = plan_step(segments, self.cache, self.vocab_size, pad_segments_to=b_pad,
-                                     fixed_max_pages=mp)
+        with trace.span("plan_step"):
+            lay, host, facts = plan_step(segments, self.cache, self.vocab_size, pad_segments_to=b_pad,
+                                         fixed_max_pages=mp)
         key = (b_pad, bucket)
         entry = self._graphs.get(key)
         if entry is None:
+            while len(self._graphs) >= max(1, int(self.cfg.max_graphs)):
+                # the least recently used shape goes: its graph, index buffers and pinned staging memory
+                # (a copy out of that memory may still run: wait for it)
+                _, old = self._graphs.popitem(last=False)
+                old.copied.synchronize()
+                torch.cuda.current_stream().synchronize()
+                old.graph = None
             entry = self._graphs[key] = _GraphEntry(b_pad, mp, self.cache.num_groups, self.rt.device)
-        full = entry.layout
-        entry.copied.synchronize()          # the previous step's copy out of the staging buffer is done
-        sn = entry.stage.numpy()
-        sn[:] = 0
-        for name in ("token_ids", "positions", "seg_of_token", "cu_q", "ctx_len", "state_slots"):
-            a, b = getattr(lay, name), getattr(full, name)
-            n = {"cu_q": b_pad + 1}.get(name, b_pad)
-            sn[b: b + n] = host[a: a + n]
-        sn[full.logit_rows: full.logit_rows + b_pad] = range(b_pad)     # every row's logits are computed
-        for g in range(self.cache.num_groups):
-            sn[full.block_tables[g]: full.block_tables[g] + b_pad * mp] = \
-                host[lay.block_tables[g]: lay.block_tables[g] + b_pad * mp]
-            sn[full.slots[g]: full.slots[g] + b_pad] = host[lay.slots[g]: lay.slots[g] + b_pad]
-        sn[entry.off_src_row: entry.off_src_row + b_pad] = -1
-        if src_rows is not None:
-            sn[entry.off_src_row: entry.off_src_row + B] = src_rows
-        if temps is not None:
-            sn[entry.off_temps: entry.off_temps + B].view(np.float32)[:] = temps
-            sn[entry.off_keys: entry.off_keys + 2 * B].view(np.int64)[:] = keys
-        entry.device_buf.copy_(entry.stage, non_blocking=True)
-        entry.copied.record()
-        if entry.graph is None:
-            facts = dict(facts, max_ctx_len=bucket)
-            ctx = context_from(full, entry.device_buf, facts)
-            ctx.src_row = entry.device_buf[entry.off_src_row: entry.off_src_row + b_pad]
-            ctx.prev_tokens = self.sampled
-            t_dev = entry.device_buf[entry.off_temps: entry.off_temps + b_pad].view(torch.float32)
-            k_dev = entry.device_buf[entry.off_keys: entry.off_keys + 2 * b_pad].view(torch.int64)
-
-            def run():
-                logits = self.model.forward(ctx, self.storage.layers)
-                ops.sample(logits, t_dev, k_dev, self.sampled[:b_pad])
-                # (dropped inside the capture, a large graph's logits go back to the pool the graphs share)
-                return logits if b_pad <= GRAPH_BATCHES[-1] else None
-            entry.runs += 1
-            logits = run()
-            if entry.runs >= 2:
-                # every library is loaded and warm by now: capture for the following steps
-                # all graphs take their intermediate buffers from one pool (they never run side by
-                # side); what a graph keeps for itself is its logits [b_pad, V], up to 256 rows
-                if self._graph_pool is None:
-                    self._graph_pool = torch.cuda.graph_pool_handle()
-                g = torch.cuda.CUDAGraph()
-                torch.cuda.synchronize()
-                with torch.cuda.graph(g, pool=self._graph_pool):
-                    entry.logits = run()
-                entry.graph = g
         else:
-            entry.graph.replay()
-            logits = entry.logits
+            self._graphs.move_to_end(key)
+        full = entry.layout
+        with trace.span("stage_copy"):
+            entry.copied.synchronize()          # the previous step's copy out of the staging buffer is done
+            sn = entry.stage.numpy()
+            sn[:] = 0
+            for name in ("token_ids", "positions", "seg_of_token", "cu_q", "ctx_len", "state_slots"):
+                a, b = getattr(lay, name), getattr(full, name)
+                n = {"cu_q": b_pad + 1}.get(name, b_pad)
+                sn[b: b + n] = host[a: a + n]
+            sn[full.logit_rows: full.logit_rows + b_pad] = range(b_pad)     # every row's logits are computed
+            for g in range(self.cache.num_groups):
+                sn[full.block_tables[g]: full.block_tables[g] + b_pad * mp] = \
+                    host[lay.block_tables[g]: lay.block_tables[g] + b_pad * mp]
+                sn[full.slots[g]: full.slots[g] + b_pad] = host[lay.slots[g]: lay.slots[g] + b_pad]
+            sn[entry.off_src_row: entry.off_src_row + b_pad] = -1
+            if src_rows is not None:
+                sn[entry.off_src_row: entry.off_src_row + B] = src_rows
+            if temps is not None:
+                sn[entry.off_temps: entry.off_temps + B].view(np.float32)[:] = temps
+                sn[entry.off_keys: entry.off_keys + 2 * B].view(np.int64)[:] = keys
+            entry.device_buf.copy_(entry.stage, non_blocking=True)
+            entry.copied.record()
+        shared = b_pad <= GRAPH_BATCHES[-1]
+        if shared and self._graph_logits is None:
+            self._graph_logits = torch.empty((GRAPH_BATCHES[-1], self.vocab_size), dtype=torch.float32,
+                                             device=self.rt.device)
+        with trace.span("launch"):
+            if entry.graph is None:
+                facts = dict(facts, max_ctx_len=bucket)
+                ctx = context_from(full, entry.device_buf, facts)
+                ctx.src_row = entry.device_buf[entry.off_src_row: entry.off_src_row + b_pad]
+                ctx.prev_tokens = self.sampled
+                # up to GRAPH_BATCHES[-1] rows the head writes into the runner's one logits buffer; a
+                # larger graph keeps none (inside the capture they go back to the pool the graphs share)
+                ctx.logits_out = self._graph_logits[:b_pad] if shared else None
+                t_dev = entry.device_buf[entry.off_temps: entry.off_temps + b_pad].view(torch.float32)
+                k_dev = entry.device_buf[entry.off_keys: entry.off_keys + 2 * b_pad].view(torch.int64)
+
+                def run():
+                    logits = self.model.forward(ctx, self.storage.layers)
+                    ops.sample(logits, t_dev, k_dev, self.sampled[:b_pad])
+                    if not shared:
+                        return None
+                    if logits.data_ptr() != self._graph_logits.data_ptr():
+                        # a head that does not write where it is told (a part that knows no `out`)
+                        self._graph_logits[:b_pad].copy_(logits)
+                    return self._graph_logits[:b_pad]
+                entry.runs += 1
+                logits = run()
+                if entry.runs >= 2:
+                    # every library is loaded and warm by now: capture for the following steps
+                    # all graphs take their intermediate buffers from one pool (they never run side by
+                    # side), and none keeps memory of its own beyond its index buffers
+                    if self._graph_pool is None:
+                        self._graph_pool = torch.cuda.graph_pool_handle()
+                    g = torch.cuda.CUDAGraph()
+                    torch.cuda.synchronize()
+                    with torch.cuda.graph(g, pool=self._graph_pool):
+                        run()
+                    entry.graph = g
+                    entry.keeps_logits = shared
+            else:
+                entry.graph.replay()
+                logits = self._graph_logits[:b_pad] if entry.keeps_logits else None
         return entry, logits, facts["ctx_lens"][:B]
 
     def _decode_step(self, segments: Sequence[Segment]):
@@ -280,7 +319,8 @@ class ModelRunner:
                 raise ValueError("only a single token can be left to the device")
             segments = [Segment(r, toks if toks[0] is not None else [0], [len(toks) - 1] if smp else [])
                         for r, toks, smp in zip(req_ids, tokens, samples)]
-            lay, host, facts = plan_step(segments, self.cache, self.vocab_size)
+            with trace.span("plan_step"):
+                lay, host, facts = plan_step(segments, self.cache, self.vocab_size)
             T, R = lay.T, lay.R
             # behind the step's own arrays: where each token comes from, and the sampling inputs
             off_src = lay.total
@@ -300,10 +340,11 @@ class ModelRunner:
             ctx = context_from(lay, dev, facts)
             ctx.src_row = dev[off_src: off_src + T]
             ctx.prev_tokens = self.sampled
-            logits = self.model.forward(ctx, self.storage.layers)
-            if R:
-                ops.sample(logits, dev[off_temps: off_temps + R].view(torch.float32),
-                           dev[off_keys: off_keys + 2 * R].view(torch.int64), self.sampled[:R])
+            with trace.span("launch"):
+                logits = self.model.forward(ctx, self.storage.layers)
+                if R:
+                    ops.sample(logits, dev[off_temps: off_temps + R].view(torch.float32),
+                               dev[off_keys: off_keys + 2 * R].view(torch.int64), self.sampled[:R])
             self._row_of = {r: i for i, r in enumerate(r for r, smp in zip(req_ids, samples) if smp)}
             if self._host_tokens is None:
                 self._host_tokens = [torch.zeros(self.sampled.numel(), dtype=torch.int32).pin_memory() for _ in range(2)]

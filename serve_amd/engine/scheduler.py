@@ -25,6 +25,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, List, Optional, Sequence
 
+from .. import trace
 from ..config.engine import EngineConfig
 from .batch import Segment
 
@@ -128,7 +129,8 @@ class Scheduler:
         """Admit the head of the queue if the policy allows it now."""
         G = self.cache.num_groups
         if self.cfg.admission == "reserve":
-            need = [self.cache.pages_for_tokens(len(r.prompt) + r.max_new_tokens)] * G
+            # what the request holds at most per group: all its tokens, or no more than a window
+            need = self._most_pages(len(r.prompt) + r.max_new_tokens)
             if any(self._reserved[g] + need[g] > self._total_pages(g) for g in range(G)):
                 return False
         else:
@@ -156,12 +158,19 @@ class Scheduler:
             self._finish(r, f"prompt ({len(r.prompt)}) + max_new_tokens ({r.max_new_tokens}) exceeds "
                             f"max_context {self.cfg.max_context}")
             return True
-        pages = self.cache.pages_for_tokens(total)
-        if any(pages > self._total_pages(g) for g in range(self.cache.num_groups)):
-            self._finish(r, f"the request needs {pages} pages, the cache has "
-                            f"{min(self._total_pages(g) for g in range(self.cache.num_groups))}")
-            return True
+        pages = self._most_pages(total)
+        for g in range(self.cache.num_groups):
+            if pages[g] > self._total_pages(g):
+                self._finish(r, f"the request needs {pages[g]} pages of cache group {g}, which has "
+                                f"{self._total_pages(g)}")
+                return True
         return False
+
+    def _most_pages(self, n_tokens: int) -> List[int]:
+        """Per cache group: the most pages a request of `n_tokens` tokens holds at any time under this
+        scheduler's portions (a group that keeps a window of keys is bounded by it)."""
+        portion = min(self.cfg.prefill_chunk, self.cfg.max_tokens_per_step)
+        return self.cache.max_pages_for(n_tokens, portion)
 
     # -- planning one step ------------------------------------------------------------------------
     def plan(self) -> StepPlan:
@@ -272,7 +281,8 @@ class Scheduler:
 
     def step(self) -> bool:
         """Plan and run one step.  False when nothing is left to do."""
-        plan = self.plan()
+        with trace.span("schedule"):
+            plan = self.plan()
         if not plan.requests:
             self._resolve()
             return False
@@ -289,20 +299,22 @@ class Scheduler:
             segments.append(Segment(r.req_id, r.tokens_between(r.fed, r.fed + n), [n - 1] if s else []))
         logits = self.runner.step(segments, borrow=True)     # sampled from before the next step
         samplers = [r for r, s in zip(plan.requests, plan.samples) if s]
-        tokens = self.sampler.sample(logits, [r.temperature for r in samplers],
-                                     [r.req_id for r in samplers], [len(r.generated) for r in samplers])
+        with trace.span("sample"):
+            tokens = self.sampler.sample(logits, [r.temperature for r in samplers],
+                                         [r.req_id for r in samplers], [len(r.generated) for r in samplers])
         self._record(plan.requests, plan.counts, samplers)
         self.steps += 1
-        for r, n in zip(plan.requests, plan.counts):
-            r.fed += n
-        for i, (r, tok) in enumerate(zip(samplers, tokens)):
-            r.generated.append(int(tok))
-            if r.keep_all_logits:
-                r.logit_rows.append(logits[i].clone())
-            if r.done() or int(tok) in self.eos:
-                if r.keep_logits:
-                    r.last_logits = logits[i].clone()
-                self._finish(r)
+        with trace.span("update_requests"):
+            for r, n in zip(plan.requests, plan.counts):
+                r.fed += n
+            for i, (r, tok) in enumerate(zip(samplers, tokens)):
+                r.generated.append(int(tok))
+                if r.keep_all_logits:
+                    r.logit_rows.append(logits[i].clone())
+                if r.done() or int(tok) in self.eos:
+                    if r.keep_logits:
+                        r.last_logits = logits[i].clone()
+                    self._finish(r)
         return True
 
     # -- decode steps with the host one step ahead ---------------------------------------------------
@@ -341,12 +353,13 @@ class Scheduler:
         previous, self._inflight = self._inflight, (handle, samplers, [len(r.generated) for r in samplers])
         self._record(reqs, plan.counts, samplers)
         self.steps += 1
-        for r, n in zip(reqs, plan.counts):
-            r.fed += n
-        for r in samplers:
-            r.generated.append(None)          # filled in when the step's tokens are read back
-            if r.done():
-                self._finish(r)
+        with trace.span("update_requests"):
+            for r, n in zip(reqs, plan.counts):
+                r.fed += n
+            for r in samplers:
+                r.generated.append(None)          # filled in when the step's tokens are read back
+                if r.done():
+                    self._finish(r)
         if previous is not None:
             self._read_back(previous)
 
@@ -359,11 +372,12 @@ class Scheduler:
         previous, self._inflight = self._inflight, (handle, list(reqs), [len(r.generated) for r in reqs])
         self._record(reqs, plan.counts, reqs)
         self.steps += 1
-        for r in reqs:
-            r.fed += 1
-            r.generated.append(None)          # filled in when the step's tokens are read back
-            if r.done():
-                self._finish(r)               # its pages may go to a later launch, which runs after this one
+        with trace.span("update_requests"):
+            for r in reqs:
+                r.fed += 1
+                r.generated.append(None)          # filled in when the step's tokens are read back
+                if r.done():
+                    self._finish(r)           # its pages may go to a later launch, which runs after this one
         if previous is not None:
             self._read_back(previous)
 

@@ -106,6 +106,36 @@ class Model:
         owners = [self._cache_owner(l) for l in self._cache_writer_layer]
         return [None if o is None else o.state_request() for o in owners]
 
+    # -- what a step costs (for measurements) ---------------------------------------------------
+    def step_cost(self, tokens: int, logit_rows: int = 1, context_before: int = 0):
+        """(elements of weights read, flops) of a step that runs `tokens` tokens of one request with
+        `context_before` tokens in the cache and computes `logit_rows` rows of logits: the parts'
+        own accounts (`Part.step_cost`) added up along the run order, so that a layer that runs
+        twice is read and computed twice.  Norms and the embedding's gathered rows count as their
+        parts say (the framework's: their weights, and nothing)."""
+        elements, flops = 0, 0.0
+        emb = self.embedding.step_cost(tokens, context_before)
+        elements, flops = elements + emb.weight_elements, flops + emb.flops
+        for e in self.spec.run_order:
+            for part in self.layers[e.layer].parts().values():
+                c = part.step_cost(tokens, context_before)
+                elements, flops = elements + c.weight_elements, flops + c.flops
+        for part, n in ((self.final_norm, logit_rows), (self.lm_head, logit_rows)):
+            c = part.step_cost(n, 0)
+            elements, flops = elements + c.weight_elements, flops + c.flops
+        return elements, flops
+
+    def cache_elements_per_token(self) -> List[Tuple[int, Optional[int]]]:
+        """Per cache layer that is read in a step (once per run-order entry that works on it):
+        (elements kept per token, window or None)."""
+        reqs = self.cache_requests()
+        out = []
+        for e in self.spec.run_order:
+            r = reqs[e.cache]
+            if r is not None:
+                out.append((sum(t.elements_per_token() for t in r.tensors), r.window))
+        return out
+
     def graph_safe(self) -> bool:
         """Whether every part only enqueues GPU work, so that a step can be captured into a graph."""
         return all(getattr(p, "graph_safe", False) for p in self._owners().values())
@@ -140,4 +170,7 @@ class Model:
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         h = self.final_norm.forward(x, pending, rows=ctx.logit_rows)
+        out = getattr(ctx, "logits_out", None)
+        if out is not None and getattr(self.lm_head, "accepts_out", False):
+            return self.lm_head.forward(h, out=out)        # the caller's buffer (a replayed step's fixed one)
         return self.lm_head.forward(h)

@@ -309,11 +309,12 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
 def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                                v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                                ctx_len: torch.Tensor, num_heads: int, scale: float, window: Optional[int],
-                               num_splits: int = 1) -> torch.Tensor:
-    """float32 attention of segments of one token each, the step's first B tokens (its tables may be
-    the head of a longer step's): a wave takes up to four query heads of a KV head, so that the keys
-    and values are read once for them.  `num_splits` > 1 cuts every key range into that many parts
-    across workgroups, merged by a second kernel."""
+                               num_splits: int = 1, first_token: int = 0) -> torch.Tensor:
+    """float32 attention of B segments of one token each, a run of the step's tokens that begins at
+    token `first_token` (the tables may be a slice of a longer step's; cu_q[i] must be first_token + i,
+    which the caller knows on the host and the kernels do not check): a wave takes up to four query
+    heads of a KV head, so that the keys and values are read once for them.  `num_splits` > 1 cuts
+    every key range into that many parts across workgroups, merged by a second kernel."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
     P, Hk, page_size, D = k_pages.shape
     _check(tiled_attention_available(q, k_pages, q_row_stride),
@@ -325,22 +326,25 @@ def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Te
     _check(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 [B, pages]")
     B = block_table.shape[0]
     _check(B <= 65535, "paged_attention_decode_f32 takes at most 65,535 segments")
-    _check(out.dim() == 2 and out.shape[0] >= B and out.shape[1] == num_heads * D and out.dtype == torch.float32,
+    rows = first_token + B
+    _check(first_token >= 0, "first_token must not be negative")
+    _check(out.dim() == 2 and out.shape[0] >= rows and out.shape[1] == num_heads * D and out.dtype == torch.float32,
            "attention output must be fp32 [T, Hq D] with a row for every segment's token")
-    _check(q.numel() >= (B - 1) * q_row_stride + num_heads * D if B else True, "q is too short")
+    _check(q.numel() >= (rows - 1) * q_row_stride + num_heads * D if B else True, "q is too short")
     _i32(cu_q, B + 1, "cu_q")
     _i32(ctx_len, B, "ctx_len")
     _check(1 <= num_splits <= 64, "num_splits out of range")
     part_o = part_ml = None
     if num_splits > 1:
-        part_o = torch.empty((B * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((B * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
+        # the parts are indexed by token, like q and out
+        part_o = torch.empty((rows * num_heads * num_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((rows * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
     lib = load_library("attention_simple")
     _ret(lib.sa_paged_attention_decode_f32(
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(num_heads), c_int(Hk), c_int(D),
-        c_int(page_size), c_float(scale), c_int(window or 0), c_int(num_splits), _ptr(part_o), _ptr(part_ml),
-        _stream()), "paged_attention_decode_f32")
+        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(first_token), c_int(num_heads),
+        c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0), c_int(num_splits), _ptr(part_o),
+        _ptr(part_ml), _stream()), "paged_attention_decode_f32")
     return out
 
 

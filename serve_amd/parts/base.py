@@ -19,7 +19,8 @@ Roles and what each must offer:
 * feed_forward  `forward(h, ctx) -> delta [T, d]`.
 * embedding     `forward(ctx) -> x` fp32 [T, d] from the step's token ids (and whatever else of
                 the step it needs: positions for a learned position table).
-* lm_head       `forward(h) -> logits` fp32 [R, V].
+* lm_head       `forward(h) -> logits` fp32 [R, V]; a head with `accepts_out = True` also takes
+                `out=`, a buffer of that shape to write them into (replayed steps bring one).
 * arrangement   puts named parts together into a layer: `PART_ROLES` (name -> role) says which
                 parts it is built from, `cache_owner()` which of them holds the layer's cache
                 and state, `forward(x, pending, ctx, cache, writes_cache) -> pending` runs it.
@@ -144,6 +145,16 @@ class Runtime:
         return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
 
 
+@dataclass
+class StepCost:
+    """What a part's share of one step costs, for measurements against the device's peaks:
+    `weight_elements`: elements of its tensors that the step reads (each once, whatever the number
+    of tokens); `flops`: multiply-adds counted as two."""
+
+    weight_elements: int = 0
+    flops: float = 0.0
+
+
 class Part:
     """Base of all parts."""
 
@@ -157,6 +168,21 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         """Receive the requested tensors (on the device, local names) and prepare for running."""
         self.rt = rt
+
+    def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
+        """The cost of running `tokens` tokens of one request that has `context_before` tokens in the
+        cache.  The default fits a part that multiplies its tokens with each of its matrices once and
+        reads every tensor it has: a part that does otherwise (a table of which rows are gathered, an
+        attention whose work grows with the context, experts of which few run) says so itself."""
+        elements, flops = 0, 0.0
+        for pr in self.param_requests():
+            n = 1
+            for d in pr.shape:
+                n *= int(d)
+            elements += n               # (a tensor that is another part's, an alias, is still read here)
+            if len(pr.shape) == 2:
+                flops += 2.0 * tokens * n
+        return StepCost(elements, flops)
 
     # mixers only
     def cache_request(self) -> Optional[TokenCacheRequest]:

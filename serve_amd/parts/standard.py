@@ -9,10 +9,10 @@ from typing import Dict, List, Optional
 
 import torch
 
-from .. import ops
+from .. import ops, trace
 from ..config.spec import PartSpec
 from ..registry import get_part, register_part
-from .base import (LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime, TokenCacheRequest,
+from .base import (LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime, StepCost, TokenCacheRequest,
                    kv_cache_request)
 from .linear import linear
 
@@ -148,6 +148,18 @@ class GQAAttention(Part):
     def cache_request(self) -> TokenCacheRequest:
         return kv_cache_request(self.num_kv_heads, self.head_dim, self.window)
 
+    def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
+        """The four projections, and scores and weighted values over the keys each token sees: token j
+        of the portion sees context_before + j + 1 keys (at most `window`), two products of head_dim
+        multiply-adds per key and query head."""
+        cost = super().step_cost(tokens, context_before)
+        if self.window:
+            keys = sum(min(context_before + j + 1, self.window) for j in range(tokens))
+        else:
+            keys = tokens * context_before + tokens * (tokens + 1) // 2
+        cost.flops += 4.0 * self.num_heads * self.head_dim * keys
+        return cost
+
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
@@ -191,10 +203,12 @@ class GQAAttention(Part):
 
     def forward(self, h: torch.Tensor, ctx, cache: LayerCache, writes_cache: bool = True) -> torch.Tensor:
         grp = ctx.groups[cache.group]
-        qkv = self._project_encode_store(h, ctx, cache, grp.slots if writes_cache else None)
+        with trace.span("write_to_cache"):                 # (with the projection and the rotation; serve/model.py:122)
+            qkv = self._project_encode_store(h, ctx, cache, grp.slots if writes_cache else None)
         attn = self.rt.empty((h.shape[0], self.num_heads * self.head_dim))
-        ops.paged_attention(qkv, qkv.shape[1], attn, cache.k_pages, cache.v_pages, grp.block_table, ctx,
-                            self.num_heads, self.scale, self.window)
+        with trace.span("attention"):                      # serve/model.py:127
+            ops.paged_attention(qkv, qkv.shape[1], attn, cache.k_pages, cache.v_pages, grp.block_table, ctx,
+                                self.num_heads, self.scale, self.window)
         return linear(attn, self.wo, partial_ok=True)      # the following norm adds the parts
 
 
@@ -252,6 +266,11 @@ class TokenEmbedding(Part):
         self.rt = rt
         self.weight = tensors["weight"]
 
+    def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
+        """A gather of `tokens` rows: no product, and of the table only those rows are read (not
+        counted: a measurement that prices a step by the tensors it streams leaves them out)."""
+        return StepCost(0, 0.0)
+
     def forward(self, ctx) -> torch.Tensor:
         """The rows of the step's tokens.  `ctx.src_row` / `ctx.prev_tokens` (when set): rows whose
         token was sampled on the device by an earlier step and never reached the host."""
@@ -283,8 +302,14 @@ class LinearHead(Part):
         self.weight = tensors["weight"]
         _prepare_products(rt, self.weight)
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return linear(h, self.weight, out_dtype=torch.float32)
+    accepts_out = True
+
+    def forward(self, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """fp32 logits [R, V]; into `out` where the caller brings the buffer."""
+        if out is not None and (out.shape != (h.shape[0], self.vocab_size) or out.dtype != torch.float32
+                                or not out.is_contiguous()):
+            raise ValueError(f"the logits buffer must be contiguous fp32 [{h.shape[0]}, {self.vocab_size}]")
+        return linear(h, self.weight, out_dtype=torch.float32, out=out)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -164,10 +164,12 @@ def next_token_of(history):
 
 
 class FakeRunner:
-    def __init__(self, num_pages, page_size, max_requests=8, max_context=256):
-        self.cache = CacheManager([None], [num_pages], page_size, max_requests, -(-max_context // page_size))
+    def __init__(self, num_pages, page_size, max_requests=8, max_context=256, windows=(None,)):
+        pools = list(num_pages) if isinstance(num_pages, (list, tuple)) else [num_pages] * len(windows)
+        self.cache = CacheManager(list(windows), pools, page_size, max_requests, -(-max_context // page_size))
         self.history = {}
         self.steps = []
+        self.most_held = [0] * len(windows)          # per group: the most pages one request held during a step
 
     def admit(self, rid):
         if self.cache.admit(rid) is None:
@@ -190,6 +192,12 @@ class FakeRunner:
                 if j in s.want:
                     out.append(next_token_of(self.history[s.req_id]))
         self.steps.append([(s.req_id, len(s.tokens)) for s in segments])
+        for s in segments:
+            for g in range(self.cache.num_groups):
+                held = sum(1 for p in self.cache.block_table(s.req_id, g) if p >= 0)
+                self.most_held[g] = max(self.most_held[g], held)
+        for s, n in zip(segments, facts["ctx_lens"]):       # as the real step does: the window moves on
+            self.cache.trim(s.req_id, n)
         self.cache.check_invariants()
         return out
 
@@ -288,6 +296,34 @@ def test_reserve_waits_for_pages_and_never_preempts():
     assert all(r.error is None and r.preemptions == 0 and r.generated == alone(r.prompt, r.max_new_tokens)
                for r in done)
     assert runner.cache.free_pages() == 12
+
+
+def test_a_windowed_group_is_reserved_by_its_window_not_by_the_whole_request():
+    """Two cache groups: one keeps every key, one a window of 8.  A request of 100 tokens needs 25 pages
+    of the first and, in portions of 8 tokens, never more than 5 of the second: with 12 pages in the
+    windowed pool, reserving admission runs two such requests side by side (counting the pages of all
+    tokens for every group would have refused each of them as larger than the pool)."""
+    ps, window, chunk = 4, 8, 8
+    cm = CacheManager([None, window], [64, 12], ps, 8, 64)
+    assert cm.max_pages_for(100, chunk) == [25, 5]
+    assert cm.max_pages_for(100, 200) == [25, 25]           # one portion holds the whole request
+    assert cm.max_pages_for(6, chunk) == [2, 2]
+    reqs = [GenerationRequest(i, [i + 1] * 60, 40) for i in range(4)]
+    runner = FakeRunner(num_pages=[64, 12], page_size=ps, windows=(None, window))
+    cfg = EngineConfig(admission="reserve", page_size=ps, num_pages=64, max_context=256, max_tokens_per_step=32,
+                       prefill_chunk=chunk)
+    sched = Scheduler(runner, FakeSampler(), cfg)
+    done = sched.run(reqs)
+    assert all(r.error is None and r.preemptions == 0 and r.generated == alone(r.prompt, r.max_new_tokens)
+               for r in done)
+    assert max(len(st) for st in runner.steps) == 2          # 2 x 25 pages of the first pool, 2 x 5 of the second
+    assert runner.most_held[0] == 25 and runner.most_held[1] <= 5
+    assert runner.cache.free_pages(0) == 64 and runner.cache.free_pages(1) == 12
+    # a request whose window alone is larger than the pool is refused, and says which group
+    small = FakeRunner(num_pages=[64, 3], page_size=ps, windows=(None, window))
+    r = GenerationRequest(0, [1] * 60, 40)
+    Scheduler(small, FakeSampler(), cfg).run([r])
+    assert r.error is not None and "group 1" in r.error and not r.generated
 
 
 def test_optimistic_preempts_the_youngest_and_tokens_do_not_change():

@@ -294,3 +294,50 @@ def test_command_line_writes_a_random_model_and_knows_the_short_names(tmp_path):
     reader = CheckpointReader(out)
     assert "model.embed_tokens.weight" in reader.names()
     assert main(["no-such-command"]) == 2
+
+
+def test_measurement_prices_a_step_by_the_parts_own_accounts():
+    """`bench.py` takes the bytes a decode step reads and the flops of a prompt from the model
+    (`Model.step_cost`, `Model.cache_elements_per_token`, which add up what each part says of itself).
+    For the dense decoder they are the sums one writes down by hand: per layer the four attention
+    matrices, the three of the feed-forward and two norm vectors; the output matrix once (tied or not:
+    the embedding's rows are gathered, not streamed) and the last norm; keys and values of every layer
+    per cached token; for a prompt of T tokens two flops per matrix element and token, the output matrix
+    for one row, and four flops per head dim, query head and visible key."""
+    import bench
+    from serve_amd.benchmark import SHAPES
+    for name in ("llama-1b", "llama-3b", "llama-8b", "tiny-a", "tiny-b"):
+        cfg = SHAPES[name]
+        model = Model(get_architecture(cfg.architecture).build_spec(cfg))
+        d, D, L = cfg.hidden_size, cfg.head_dim, cfg.num_hidden_layers
+        matrices = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D * d + d * cfg.num_attention_heads * D
+                    + 3 * d * cfg.intermediate_size)
+        assert bench.weight_bytes(model, 2) == 2 * ((matrices + 2 * d) * L + cfg.vocab_size * d + d)
+        assert bench.kv_bytes(model, 384, 2) == 384 * 2 * L * cfg.num_key_value_heads * D * 2
+        T = 2048
+        want = 2.0 * matrices * L * T + 2.0 * cfg.vocab_size * d + 4.0 * cfg.num_attention_heads * D * L * (T * (T + 1) / 2)
+        assert bench.prefill_flops(model, T) == want
+    assert bench.weight_bytes(Model(get_architecture("LlamaForCausalLM").build_spec(SHAPES["llama-1b"])), 2) == 2471628800
+    # a portion over earlier keys, and a window: the attention's own account
+    from serve_amd.parts.standard import GQAAttention
+    from serve_amd.config.spec import PartSpec
+    pos = PartSpec("rope", {"head_dim": 16, "rot_dim": 16, "theta": 10000.0})
+    proj = 2.0 * 5 * (64 * 64 + 2 * 32 * 64 + 64 * 64)
+    full = GQAAttention(64, 4, 2, 16, 0.25, pos).step_cost(5, context_before=10)
+    assert full.flops == proj + 4.0 * 4 * 16 * (11 + 12 + 13 + 14 + 15)
+    windowed = GQAAttention(64, 4, 2, 16, 0.25, pos, window=12).step_cost(5, context_before=10)
+    assert windowed.flops == proj + 4.0 * 4 * 16 * (11 + 12 + 12 + 12 + 12)
+
+
+def test_float32_products_of_a_few_dozen_rows_leave_no_part_of_k_without_stages():
+    """The float32 product for 9 to 128 rows cuts its inner dimension into parts across workgroups, in
+    stages of 256 columns spread evenly: with no more parts than stages no part is empty (an empty part
+    stores zeros and reads the matrix's last stage, in range; this only says that none is chosen)."""
+    from serve_amd import ops
+    for K in (512, 1024, 2048, 2304, 3072, 4096, 5120, 8192, 14336):
+        for N in (512, 1024, 2048, 2304, 3072, 4096):
+            for M in (9, 16, 64, 65, 128):
+                parts = ops.f32_mid_parts(M, N, K)
+                stages = -(-K // 256)
+                assert 1 <= parts <= 8 and parts <= stages
+                assert all((z + 1) * stages // parts - z * stages // parts >= 1 for z in range(parts))

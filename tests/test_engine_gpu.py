@@ -17,7 +17,8 @@ DTYPES = ["float32", "bfloat16"]
 # order one and the bfloat16 runs can fail on the rotation, the score scale and the head mapping;
 # 32: tensors stored in float32 (the float32 engine then computes on weights that bfloat16 cannot
 # hold; the bfloat16 engine keeps them 32-bit and multiplies bfloat16 activations with them)
-MODELS = ["A", "B", "C", "AS", "BS", "CS", "A32", "B32", "BS32"]
+# B512: Tiny B with the vocabulary it is specified with (the `tiny-b` shape of serve_amd.benchmark)
+MODELS = ["A", "B", "C", "AS", "BS", "CS", "A32", "B32", "BS32", "B512"]
 
 
 def engine_for(tmp_path, name, dtype, num_pages=64, page_size=8, **kw):

@@ -403,8 +403,9 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     """A mixer that keeps, per request, the running sum of the activations it has seen
     (out[t] = proj(sum of h[0..t])): state of fixed size, no paged cache.  It lives in this test
     only; the framework's files are not touched.  Fed whole or in portions, beside another
-    request, its logits must be the same, which needs the state slots to be zeroed at admission,
-    kept between steps and separated between requests."""
+    request, its logits must be those of the same model written in plain torch (float64, whole
+    sequence), which needs the state slots to be zeroed at admission, kept between steps and
+    separated between requests."""
     from dataclasses import dataclass
 
     import serve_amd
@@ -494,6 +495,22 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         eng.runner.release("w")
         return out
     wa, wb = whole(a), whole(b)
+
+    def plain(tokens):
+        """The same model in plain torch, float64, whole sequence: the oracle of the engine's runs."""
+        w = {k: v.double() for k, v in util.plain_weights(folder).items()}
+
+        def norm(x, g):
+            return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-5) * g
+        x = w["toy.embed"][torch.tensor(tokens)]
+        for i in range(2):
+            p = f"toy.{i}."
+            x = x + torch.cumsum(norm(x, w[p + "n1"]), dim=0) @ w[p + "proj"].T
+            h = norm(x, w[p + "n2"])
+            x = x + (torch.nn.functional.silu(h @ w[p + "gate"].T) * (h @ w[p + "up"].T)) @ w[p + "down"].T
+        return norm(x, w["toy.norm"]) @ w["toy.embed"].T
+    torch.testing.assert_close(wa.double().cpu(), plain(a), atol=2e-5, rtol=1e-4)
+    torch.testing.assert_close(wb.double().cpu(), plain(b), atol=2e-5, rtol=1e-4)
     eng.runner.admit("a")
     eng.runner.admit("b")
     r1 = eng.step([Segment("a", a[:5], list(range(5))), Segment("b", b[:1], [0])])
@@ -515,7 +532,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     def greedy(tokens, n):
         seq, new = list(tokens), []
         for _ in range(n):
-            t = int(whole(seq)[-1].argmax())
+            t = int(plain(seq)[-1].argmax())
             new.append(t)
             seq.append(t)
         return new

@@ -748,3 +748,140 @@ def test_memory_ceiling_kernels_copy_and_refuse():
         ops.read_bytes(torch.zeros(24, dtype=torch.uint8, device=DEV))
     with pytest.raises(ops.KernelError):
         ops.copy_bytes(torch.zeros(32, dtype=torch.uint8, device=DEV), torch.zeros(48, dtype=torch.uint8, device=DEV))
+
+
+# ---------------------------------------------------------------------------------------------
+# attention at the contexts whose speeds are published: thousands to a hundred thousand keys
+# ---------------------------------------------------------------------------------------------
+def long_context_case(dtype, segs, kernel, splits, seed, Hq=32, Hk=8, D=64, ps=16, mode="edges"):
+    """segs: (ctx_before, q_len) at contexts of thousands of keys, pages shuffled.  With random keys a
+    softmax over that many of them is an average in which one lost or doubled block of keys drowns, so
+    the data are made to show it.  mode "edges": all keys are small but about two dozen per segment
+    and KV head, drawn from the ends of the context, the edges of blocks of 32 and 64 keys and of every
+    part a split key range could have, and random places; those stand out by a score of about 14 with
+    slightly different heights, so that each carries a few percent of the weight and its value row
+    moves the output by more than the tolerance when it is missed, taken twice or taken from the wrong
+    place.  mode "random": scores with a spread of 3.5, so that in every (segment, head) a few keys at
+    random places carry the weight."""
+    from types import SimpleNamespace
+
+    from serve_amd import ops
+    rng = random.Random(seed)
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    B, T = len(segs), sum(q for _, q in segs)
+    G = Hq // Hk
+    ctxs = [c + q for c, q in segs]
+    MP = -(-max(ctxs) // ps)
+    P = sum(-(-n // ps) for n in ctxs) + 5
+    order = torch.randperm(P, generator=g, device=DEV)
+    edges = mode == "edges"
+    k_pages = (torch.randn((P, Hk, ps, D), generator=g, device=DEV) * (0.1 if edges else 1.0)).to(DT[dtype])
+    v_pages = torch.randn((P, Hk, D, ps), generator=g, device=DEV).to(DT[dtype])
+    u = torch.nn.functional.normalize(torch.randn((Hk, D), generator=g, device=DEV), dim=-1) * math.sqrt(D)
+    bt = torch.zeros((B, MP), dtype=torch.int32, device=DEV)
+    q = torch.empty((T, Hq, D), dtype=DT[dtype], device=DEV)
+    at, row = 0, 0
+    for i, (c, ql) in enumerate(segs):
+        n = ctxs[i]
+        npages = -(-n // ps)
+        mine = order[at: at + npages]
+        at += npages
+        bt[i, :npages] = mine.int()
+        if not edges:
+            q[row: row + ql] = (torch.randn((ql, Hq, D), generator=g, device=DEV) * 3.5).to(DT[dtype])
+            row += ql
+            continue
+        always = {0, n - 1, c}
+        cand = {1, n - 2, n // 2, 31, 32, 63, 64, max(c - 1, 0)}
+        for parts in (2, 3, 4, 8, 16, 64):
+            for j in range(1, parts, max(1, parts // 4)):
+                e = (n * j) // parts
+                cand.update({e - 1, e, 32 * (e // 32), 32 * (e // 32) - 1, 64 * (e // 64), 64 * (e // 64) - 1})
+        cand.update(rng.randrange(n) for _ in range(12))
+        cand = sorted(p for p in cand if 0 <= p < n and p not in always)
+        special = sorted(always) + rng.sample(cand, min(len(cand), 45))
+        pos = torch.tensor(special, device=DEV)
+        height = 1.5 + 0.06 * torch.rand((len(special), Hk, 1), generator=g, device=DEV)
+        # every KV head gets its own half of them (and all get the context's ends)
+        chosen = torch.rand((len(special), Hk, 1), generator=g, device=DEV) < 0.5
+        chosen[: len(always)] = True
+        old = k_pages[mine[pos // ps], :, pos % ps, :]
+        k_pages[mine[pos // ps], :, pos % ps, :] = torch.where(chosen, (u[None] * height).to(DT[dtype]), old)
+        # queries along the same direction: score = q.k / sqrt(D) = sqrt(D) * 1.17 * 1.5 = 14 for the chosen keys
+        noise = torch.randn((ql, Hq, D), generator=g, device=DEV) * 0.3
+        q[row: row + ql] = (u.repeat_interleave(G, dim=0)[None] * 1.17 + noise).to(DT[dtype])
+        row += ql
+    q = q.view(T, Hq * D)
+    cu = [0]
+    for _, ql in segs:
+        cu.append(cu[-1] + ql)
+    cu_q = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    ctx_len = torch.tensor(ctxs, dtype=torch.int32, device=DEV)
+    out = torch.full((T, Hq * D), float("nan"), dtype=DT[dtype], device=DEV)
+    scale = D ** -0.5
+    max_q = max(ql for _, ql in segs)
+    if kernel == "mfma":
+        ops.paged_attention_mfma(q, Hq * D, out, k_pages, v_pages, bt, cu_q, ctx_len, T, max_q, Hq, scale, None, splits)
+    elif kernel == "decode_f32":
+        ops.paged_attention_decode_f32(q, Hq * D, out, k_pages, v_pages, bt, cu_q, ctx_len, Hq, scale, None, splits)
+    else:
+        seg_of = torch.tensor([i for i, (_, ql) in enumerate(segs) for _ in range(ql)], dtype=torch.int32, device=DEV)
+        ctx = SimpleNamespace(num_segments=B, num_tokens=T, cu_q=cu_q, ctx_len=ctx_len, seg_of_token=seg_of,
+                              q_lens=[ql for _, ql in segs], ctx_lens=ctxs, max_q_len=max_q, max_ctx_len=max(ctxs),
+                              decode_only=max_q == 1)
+        ops.paged_attention(q, Hq * D, out, k_pages, v_pages, bt, ctx, Hq, scale, None)
+        if splits:          # what the dispatcher is expected to choose for this launch
+            assert ops.attention_splits(max_q, B, Hk, max(ctxs), G) == splits or dtype == "float32"
+    # dense softmax in float64, one KV head at a time
+    row = 0
+    for i, (c, ql) in enumerate(segs):
+        n = ctxs[i]
+        npages = -(-n // ps)
+        pages = bt[i, :npages].long()
+        qi = q[row: row + ql].double().view(ql, Hk, G, D)
+        qpos = torch.arange(c, c + ql, device=DEV)[:, None]
+        vis = (torch.arange(n, device=DEV)[None, :] <= qpos)[:, None, :]
+        for h in range(Hk):
+            K = k_pages[pages, h].double().reshape(npages * ps, D)[:n]
+            V = v_pages[pages, h].double().permute(0, 2, 1).reshape(npages * ps, D)[:n]
+            s = torch.einsum("qgd,kd->qgk", qi[:, h], K) * scale
+            s = s.masked_fill(~vis, float("-inf"))
+            want = torch.einsum("qgk,kd->qgd", torch.softmax(s, -1), V)
+            got = out[row: row + ql].double().view(ql, Hk, G, D)[:, h]
+            torch.testing.assert_close(got, want, **tol(dtype),
+                                       msg=lambda m: f"segment {i} {segs[i]}, KV head {h}, {splits} splits: {m}")
+        row += ql
+
+
+@pytest.mark.parametrize("dtype,kernel", [("bfloat16", "mfma"), ("float32", "decode_f32")])
+@pytest.mark.parametrize("contexts,splits", [
+    ([4096, 4095, 4097, 4081, 3950, 4100, 2047, 4096], 8),      # the measured configuration: batch 8, 8 key splits
+    ([4096, 4033, 1], 64),
+    ([32768, 32767, 30001], 8), ([32768, 20000], 64),
+    ([131072, 100001], 64), ([131071], 8)])
+def test_decode_attention_at_long_contexts(dtype, kernel, contexts, splits):
+    """Single decoded tokens at head size 64, four query heads per KV head, page size 16, over 4,096,
+    32,768 and 131,072 keys with 8 and 64 parts of the key range: the configurations whose speeds are
+    measured, in bfloat16 (matrix cores) and float32."""
+    segs = [(n - 1, 1) for n in contexts]
+    long_context_case(dtype, segs, kernel, splits, seed=700 + len(contexts) + splits)
+    long_context_case(dtype, segs, kernel, splits, seed=750 + len(contexts) + splits, mode="random")
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_decode_attention_at_long_contexts_as_the_engine_calls_it(dtype):
+    """The same through the dispatcher, which chooses the number of parts itself: batch 8 at 4,096
+    keys (8 parts on 256 compute units), batch 64 at 4,096, batch 8 at 32,768."""
+    long_context_case(dtype, [(4095 - 3 * i, 1) for i in range(8)], "dispatch", 8, seed=731)
+    long_context_case(dtype, [(4095 - 17 * i, 1) for i in range(64)], "dispatch", 0, seed=732)
+    long_context_case(dtype, [(32767 - 1001 * i, 1) for i in range(8)], "dispatch", 8, seed=733)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_prompt_portion_over_a_long_context(dtype):
+    """A portion of 2,048 tokens of a long prompt over 30,000 earlier keys, as the engine calls it (the
+    key range cut across workgroups, since the portion is a small share of its context), and a portion
+    of 600 tokens over 9,000 beside it; fewer heads than the measured shape to keep the dense softmax small."""
+    long_context_case(dtype, [(30000, 2048)], "dispatch", 0, seed=741, Hq=8, Hk=2)
+    long_context_case(dtype, [(30000, 2048)], "dispatch", 0, seed=743, Hq=8, Hk=2, mode="random")
+    long_context_case(dtype, [(9000, 600), (30000, 1), (12001, 130)], "dispatch", 0, seed=742, Hq=8, Hk=2)

@@ -141,12 +141,200 @@ def test_more_than_256_requests_decode_from_a_graph_that_keeps_no_logits(tmp_pat
     big = [st for st in log if len(st["requests"]) > 256 and set(st["counts"]) == {1}]
     assert len(big) >= 4, "no decode steps of more than 256 requests were run"
     entry = engine.runner._graphs.get((384, 256))
-    assert entry is not None and entry.graph is not None and entry.logits is None
+    assert entry is not None and entry.graph is not None and not entry.keeps_logits
     assert all(o.error is None and len(o.generated_tokens) == new for o in out)
     for i in list(range(0, count, 13)) + [count - 1]:
         check_tokens(folder, prompts[i], out[i].generated_tokens.tolist(), dtype, f"request {i} of {count}",
                      temperature=temps[i], rid=i)
     engine.runner.cache.check_invariants()
+
+
+_PLAIN_CACHE = {}
+
+
+def plain_tail(folder, name, tokens, first):
+    """The plain model's logits from position `first` on; kept, so that the two dtypes share the run."""
+    key = (name, tuple(tokens), first)
+    if key not in _PLAIN_CACHE:
+        _PLAIN_CACHE[key] = util.plain_logits(folder, tokens)[first:].clone()
+    return _PLAIN_CACHE[key]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_decode_across_4096_keys(tmp_path, dtype):
+    """The measured configuration in small: eight requests at head size 64 with four query heads per
+    KV head and pages of 16 tokens are decoded for 40 steps while their contexts pass 4,096 tokens:
+    graphs of batch 8 for the buckets up to 4,096 and up to 8,192 keys (eight and more parts of the key
+    range, merged), every logit against the plain model."""
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.runner import GRAPH_BATCHES
+    name, count, steps = "CS", 8, 40
+    folder = util.make_folder(tmp_path, name)
+    vocab = util.tiny_config(name).vocab_size
+    rng = random.Random(41)
+    lens = [4096 - 21 + 2 * i for i in range(count)]          # 4,075 .. 4,089: all pass 4,096 within the 40 steps
+    tokens = [util.random_tokens(rng, n + steps, vocab) for n in lens]
+    engine = make_engine(folder, dtype, page_size=16, num_pages=count * 260, max_context=8192, max_requests=count,
+                         max_tokens_per_step=8192, prefill_chunk=8192)
+    runner = engine.runner
+    for i in range(count):
+        assert runner.admit(i)
+        engine.step([Segment(i, tokens[i][: lens[i]], [])])
+    got = [[] for _ in range(count)]
+    for s in range(steps):
+        logits = engine.step([Segment(i, [tokens[i][lens[i] + s]], [0]) for i in range(count)])
+        for i in range(count):
+            got[i].append(logits[i])
+    assert 8 in GRAPH_BATCHES
+    for bucket in (4096, 8192):
+        entry = runner._graphs.get((8, bucket))
+        assert entry is not None and entry.graph is not None, f"no graph was replayed for batch 8, bucket {bucket}"
+    for i in range(count):
+        want = plain_tail(folder, name, tokens[i], lens[i])
+        util.assert_close(torch.stack(got[i]), want, dtype, f"{name} {dtype} request {i} across 4,096 keys")
+        runner.release(i)
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_600_live_requests_step_beyond_the_largest_graph(tmp_path, dtype):
+    """600 requests live at once through the entry point: their decode steps have more than 512
+    single-token rows, more than any graph takes, and are launched kernel by kernel ahead of the host;
+    the tokens of a sample of the requests are the plain model's."""
+    from serve_amd.engine.engine import Request
+    from serve_amd.engine.runner import ASYNC_GRAPH_BATCHES
+    folder = util.make_folder(tmp_path, "AS")
+    vocab = util.tiny_config("AS").vocab_size
+    rng = random.Random(43)
+    count, new = 600, 6
+    prompts = [util.random_tokens(rng, rng.randrange(3, 9), vocab) for _ in range(count)]
+    engine = make_engine(folder, dtype, page_size=8, num_pages=count * 3, max_context=64, max_requests=count,
+                         max_tokens_per_step=8192, prefill_chunk=64, seed=SEED)
+    log = []
+    temps = [0.0 if i % 3 else 0.7 for i in range(count)]
+    out = engine.generate([Request(torch.tensor(p), len(p), new) for p in prompts], temperature=temps, step_log=log)
+    big = [st for st in log if len(st["requests"]) > ASYNC_GRAPH_BATCHES[-1] and set(st["counts"]) == {1}]
+    assert len(big) >= 4, "no decode steps of more than 512 requests were run"
+    assert engine.runner._eager_launches >= len(big)
+    assert all(o.error is None and len(o.generated_tokens) == new for o in out)
+    for i in list(range(0, count, 29)) + [count - 1]:
+        check_tokens(folder, prompts[i], out[i].generated_tokens.tolist(), dtype, f"request {i} of {count}",
+                     temperature=temps[i], rid=i)
+    engine.runner.cache.check_invariants()
+    assert not engine.runner.cache.live_requests()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_admission_in_turns_on_the_device(tmp_path, dtype):
+    """`admit_interval` 4 with six slots for thirty requests: newcomers start only every fourth step
+    while others run, the steps between are decode steps replayed from graphs and launched ahead of
+    the host, and every request's tokens are the plain model's."""
+    from serve_amd.engine.engine import Request
+    folder = util.make_folder(tmp_path, "AS")
+    vocab = util.tiny_config("AS").vocab_size
+    rng = random.Random(44)
+    count = 30
+    prompts = [util.random_tokens(rng, rng.randrange(2, 12), vocab) for _ in range(count)]
+    new = [rng.randrange(1, 10) for _ in range(count)]
+    engine = make_engine(folder, dtype, page_size=8, num_pages=64, max_context=64, max_requests=6,
+                         max_tokens_per_step=64, prefill_chunk=16, admit_interval=4, seed=SEED)
+    log = []
+    out = engine.generate([Request(torch.tensor(p), len(p), n) for p, n in zip(prompts, new)], step_log=log)
+    started, starts = set(), []
+    for i, st in enumerate(log):
+        fresh = [r for r in st["requests"] if r not in started]
+        if fresh:
+            starts.append((i, len(st["requests"]) - len(fresh)))
+        started.update(fresh)
+    for (a, _), (b, others) in zip(starts, starts[1:]):
+        assert b - a >= 4 or others == 0, f"newcomers at steps {a} and {b} with {others} others running"
+    assert sum(e.launches for e in engine.runner._graphs.values()) > 0, "no decode step ran from a graph"
+    for i, (p, n, r) in enumerate(zip(prompts, new, out)):
+        assert r.error is None and len(r.generated_tokens) == n
+        check_tokens(folder, p, r.generated_tokens.tolist(), dtype, f"request {i} admitted in turns", rid=i)
+    engine.runner.cache.check_invariants()
+
+
+def test_graph_memory_is_bounded(tmp_path):
+    """Decode steps of six batch sizes with a vocabulary of 32,000: all graphs write their logits into
+    one buffer of the runner, so the device's free memory stops falling once the largest shape has been
+    captured (a buffer per graph would take 98 MB more here), and with `max_graphs` 3 the least recently
+    used shapes are dropped and captured again when they come back, with the same logits."""
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.llama import LlamaConfig
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    cfg = LlamaConfig(vocab_size=32000, hidden_size=64, intermediate_size=128, num_hidden_layers=1,
+                      num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-5,
+                      rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True)
+    engine = Engine.from_config(cfg, seed=3, cfg=EngineConfig(dtype="bfloat16", page_size=16, num_pages=600,
+                                                               max_context=64, max_requests=256, max_graphs=3))
+    runner = engine.runner
+    rng = random.Random(51)
+    ids = list(range(200))
+    for i in ids:
+        assert runner.admit(i)
+    engine.step([Segment(i, util.random_tokens(rng, 3, cfg.vocab_size), []) for i in ids])
+
+    def decode(n):
+        """Three steps of the first n requests with the same tokens: eager, eager + capture, replay.  The
+        logits of a step depend on its tokens and their contexts, which grow by one each step."""
+        return [engine.step([Segment(i, [7 + i], [0]) for i in ids[:n]]) for _ in range(3)]
+    dev = runner.rt.device
+    decode(200)                                    # padded to 256 rows: the largest shape comes first
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info(dev)[0]
+    for n in (130, 100, 90, 70, 50):               # 160, 112, 96, 80 and 64 rows
+        decode(n)
+        assert len(runner._graphs) <= 3
+    torch.cuda.synchronize()
+    fallen = free0 - torch.cuda.mem_get_info(dev)[0]
+    assert fallen <= 16 << 20, f"free memory fell by {fallen >> 20} MB while five more shapes were captured"
+    assert [k[0] for k in runner._graphs] == [96, 80, 64]          # the three most recently used
+    assert all(e.graph is not None and e.keeps_logits for e in runner._graphs.values())
+    # a shape that was dropped comes back: captured again, and what it computes is what a step computes
+    # that is launched kernel by kernel
+    got = decode(130)[2]
+    assert (160, 256) in runner._graphs and runner._graphs[(160, 256)].graph is not None
+    for i in ids:
+        runner.release(i)
+    eager = Engine.from_config(cfg, seed=3, cfg=EngineConfig(dtype="bfloat16", page_size=16, num_pages=600,
+                                                              max_context=64, max_requests=256, use_graphs=False))
+    # the same history without graphs: prompts, then the same single tokens for as many steps
+    rng = random.Random(51)
+    for i in ids:
+        assert eager.runner.admit(i)
+    eager.step([Segment(i, util.random_tokens(rng, 3, cfg.vocab_size), []) for i in ids])
+    last = None
+    for n, times in ((200, 3), (130, 3), (100, 3), (90, 3), (70, 3), (50, 3), (130, 3)):
+        for _ in range(times):
+            last = eager.step([Segment(i, [7 + i], [0]) for i in ids[:n]])
+    assert (got - last).abs().max().item() <= 4e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_poisoned_cache_changes_nothing(tmp_path, dtype):
+    """The debugging mode in which every page of the cache holds NaN until a token is stored in it and
+    again once it is given back: with so few pages that they are used again, prompt portions beside
+    decoding requests, every logit is finite and the tokens are those of the ordinary run."""
+    from serve_amd.engine.engine import Request
+    folder = util.make_folder(tmp_path, "CS")
+    vocab = util.tiny_config("CS").vocab_size
+    rng = random.Random(52)
+    prompts = [util.random_tokens(rng, rng.randrange(2, 60), vocab) for _ in range(14)]
+    reqs = [Request(torch.tensor(p), len(p), 9) for p in prompts]
+    kw = dict(page_size=16, num_pages=24, max_context=128, max_requests=5, max_tokens_per_step=40, prefill_chunk=24)
+    plain_run = make_engine(folder, dtype, **kw).generate(reqs, return_logits="all")
+    engine = make_engine(folder, dtype, debug_poison_cache=True, **kw)
+    assert torch.isnan(engine.runner.storage.layers[0].k_pages).all()
+    out = engine.generate(reqs, return_logits="all")
+    for i, (a, b) in enumerate(zip(plain_run, out)):
+        assert b.error is None and torch.isfinite(b.logits).all(), f"request {i}: a logit is not finite"
+        assert a.generated_tokens.tolist() == b.generated_tokens.tolist(), f"request {i}"
+        assert (a.logits - b.logits).abs().max().item() == 0.0
+    # everything was given back, so everything is poisoned again
+    assert torch.isnan(engine.runner.storage.layers[0].k_pages).all()
+    assert torch.isnan(engine.runner.storage.layers[1].v_pages).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -7,6 +7,7 @@ vocabulary (256 / 509, the second odd), rope theta and llama3 scaling, eps, tied
 """
 from __future__ import annotations
 
+import dataclasses
 import json
 import os
 import random
@@ -39,6 +40,10 @@ TINY_C = LlamaConfig(vocab_size=1000, hidden_size=192, intermediate_size=320, nu
 
 TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 
+# Tiny B as it is specified (the `tiny-b` shape): the same but for the vocabulary, 512 instead of the
+# odd 509 that most tests use to reach the unaligned stores of the output product
+TINY_B512 = dataclasses.replace(TINY_B, vocab_size=512)
+
 # Tolerances on logits against the plain fp64 model.  Logits of these models are O(0.1..1).
 # float32: every operation is fp32 with fp32 accumulation, so errors are a few ulp of the
 # largest intermediate.  bfloat16: weights are exact (stored bf16), activations are rounded to
@@ -55,13 +60,18 @@ SHARP_SCALES = {r"self_attn\.(q|k)_proj": 4.0}
 
 
 def tiny_config(name: str):
-    """name = A, B or C, then S for the sharp variant, then 32 for tensors stored in float32."""
+    """name = A, B or C (or B512: Tiny B with its specified vocabulary), then S for the sharp variant,
+    then 32 for tensors stored in float32."""
+    if name == "B512":
+        return TINY_B512
     return TINY[name[0]][0]
 
 
 def make_folder(tmp_path, name: str) -> str:
     cfg, seed = TINY[name[0]]
     rest = name[1:]
+    if name == "B512":
+        cfg, rest = TINY_B512, ""
     sharp = rest.startswith("S")
     stored = torch.float32 if rest.endswith("32") else torch.bfloat16
     assert rest in ("", "S", "32", "S32"), name

@@ -176,7 +176,8 @@ def measured_ceilings():
 def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
     """`--report`: every number of the measurement with the bytes or flops it stands for, as a
     share of the published peaks and of the ceilings measured on this device.  With `make_engine`
-    (context -> engine) also decode steps at contexts of 32k and 128k tokens."""
+    (batch, context[, dtype] -> engine) also decode steps at batch 1 and 64 at the headline's context, at
+    contexts of 32k and 128k tokens, and the float32 path at the headline's batch and context."""
     import torch
     ceil = measured_ceilings()
     print(f"measured ceilings: own read kernel {ceil['own_read'] / 1e12:.2f} TB/s, own copy kernel "
@@ -204,11 +205,19 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
     if make_engine is not None:
         del engine
         torch.cuda.empty_cache()
-        for batch, context in ((8, 32768), (64, 32768), (8, 131072)):
+        # the context that the headline is measured at, at the other batch sizes; then longer contexts
+        for batch, context in ((1, 4096), (64, 4096), (8, 32768), (64, 32768), (8, 131072)):
             eng = make_engine(batch, context)
             decode_row(eng, batch, context - 64 - 16 - 3 - head_start(eng, batch, context), 16, 64)
             del eng
             torch.cuda.empty_cache()
+        # the true 32-bit path at the headline's batch and context: twice the bytes, the same kernels' float32 kin
+        eng = make_engine(8, 4096, "float32")
+        dt, mean_ctx = decode_run(eng, 8, 4096 - 64 - 16 - 3 - head_start(eng, 8, 4096), 16, 64, seed=28)
+        nbytes = weight_bytes(eng.model, 4) + 8 * kv_bytes(eng.model, mean_ctx, 4)
+        rate = nbytes / (dt / 64)
+        print(f"{f'float32 decode, batch 8, context ~{int(mean_ctx)}':34s} {dt / 64 * 1e3:8.3f} {8 * 64 / dt:10.0f} "
+              f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}", flush=True)
     return 0
 
 
@@ -268,11 +277,12 @@ def main() -> int:
                                       "frac": round(prefill_flops(engine.model, T) / pt / peak, 4)}}), flush=True)
         return 0
     if args.report:
-        def long_engine(batch, context):
+        def long_engine(batch, context, dtype="bfloat16"):
             pages = batch * (-(-context // page)) + 64
             return Engine.from_config(cfg, seed=0, cfg=EngineConfig(
-                dtype="bfloat16", page_size=page, num_pages=pages, max_context=context, max_requests=batch,
-                max_tokens_per_step=2048 + batch, prefill_chunk=2048, admission="reserve"))
+                dtype=dtype, page_size=page, num_pages=pages, max_context=context, max_requests=batch,
+                max_tokens_per_step=2048 + batch, prefill_chunk=2048, admission="reserve"),
+                weight_dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32)
         return report(engine, cfg, args.steps, args.warmup, long_engine)
     steps, warmup = args.steps, args.warmup
     prompt_len = args.context - (warmup + steps + 3) - head_start(engine, args.batch, args.context)

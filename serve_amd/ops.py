@@ -8,7 +8,8 @@ library that cannot be compiled is an error (`serve_amd.csrc.build.BuildError`).
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from dataclasses import dataclass
+from typing import Optional, Sequence
 
 import torch
 
@@ -695,6 +696,25 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
 # dispatch between kernels of the same operation
 # ---------------------------------------------------------------------------------------------
 
+@dataclass
+class AttentionStep:
+    """What `paged_attention` needs to know of a step: the segments' token offsets and context lengths
+    on the device, and the same facts on the host so that choosing kernels and grids needs no
+    read-back.  The engine's `StepContext` has these attributes and is passed as it is; a mixer that
+    brings its own segment layout (tokens of its own, another notion of a request) fills one of these."""
+
+    num_segments: int
+    num_tokens: int
+    cu_q: torch.Tensor               # int32 [B + 1]: first token of every segment, and the end
+    ctx_len: torch.Tensor            # int32 [B]: keys a segment's last token sees (its context after the step)
+    seg_of_token: torch.Tensor       # int32 [T]
+    q_lens: Sequence[int]            # the host's copies
+    ctx_lens: Sequence[int]
+    max_q_len: int
+    max_ctx_len: int
+    decode_only: bool = False
+
+
 def _attention_launches(ctx):
     """How a step's segments go to the matrix-core attention kernels.  Single decoded tokens take
     the one-wave kernel and a split key range, prompt portions the kernel that shares keys and
@@ -723,9 +743,10 @@ def _attention_launches(ctx):
 def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                     v_pages: torch.Tensor, block_table: torch.Tensor, ctx, num_heads: int, scale: float,
                     window: Optional[int]) -> torch.Tensor:
-    """Attention over the paged cache for all tokens of the step described by `ctx`
-    (`serve_amd.engine.batch.StepContext`): the matrix-core kernel for bf16 where it takes the
-    sizes, else the general fp32-arithmetic kernel."""
+    """Attention over the paged cache for all tokens of the step described by `ctx` (an `AttentionStep`,
+    or anything with its attributes: the engine passes its `StepContext`): the matrix-core kernel for
+    bf16 where it takes the sizes, else the general fp32-arithmetic kernel.  The plan of launches is
+    kept on `ctx`, so that the layers of a step share it."""
     if mfma_attention_available(q, k_pages, q_row_stride, scale):
         Hk = k_pages.shape[1]
         # (first segment, segments, tokens up to their end, longest portion, longest context)

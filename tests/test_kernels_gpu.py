@@ -763,8 +763,6 @@ def long_context_case(dtype, segs, kernel, splits, seed, Hq=32, Hk=8, D=64, ps=1
     moves the output by more than the tolerance when it is missed, taken twice or taken from the wrong
     place.  mode "random": scores with a spread of 3.5, so that in every (segment, head) a few keys at
     random places carry the weight."""
-    from types import SimpleNamespace
-
     from serve_amd import ops
     rng = random.Random(seed)
     g = torch.Generator(device=DEV).manual_seed(seed)
@@ -826,9 +824,10 @@ def long_context_case(dtype, segs, kernel, splits, seed, Hq=32, Hk=8, D=64, ps=1
         ops.paged_attention_decode_f32(q, Hq * D, out, k_pages, v_pages, bt, cu_q, ctx_len, Hq, scale, None, splits)
     else:
         seg_of = torch.tensor([i for i, (_, ql) in enumerate(segs) for _ in range(ql)], dtype=torch.int32, device=DEV)
-        ctx = SimpleNamespace(num_segments=B, num_tokens=T, cu_q=cu_q, ctx_len=ctx_len, seg_of_token=seg_of,
-                              q_lens=[ql for _, ql in segs], ctx_lens=ctxs, max_q_len=max_q, max_ctx_len=max(ctxs),
-                              decode_only=max_q == 1)
+        # (a caller outside the engine describes its step with ops.AttentionStep)
+        ctx = ops.AttentionStep(num_segments=B, num_tokens=T, cu_q=cu_q, ctx_len=ctx_len, seg_of_token=seg_of,
+                                q_lens=[ql for _, ql in segs], ctx_lens=ctxs, max_q_len=max_q, max_ctx_len=max(ctxs),
+                                decode_only=max_q == 1)
         ops.paged_attention(q, Hq * D, out, k_pages, v_pages, bt, ctx, Hq, scale, None)
         if splits:          # what the dispatcher is expected to choose for this launch
             assert ops.attention_splits(max_q, B, Hk, max(ctxs), G) == splits or dtype == "float32"

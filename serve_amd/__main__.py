@@ -46,6 +46,9 @@ def _generate(argv) -> int:
                     "others run, so that the steps between are pure decode steps (1: at every step)")
     ap.add_argument("--max-graphs", type=int, default=64, help="captured decode steps kept (one per padded batch "
                     "size and bucket of contexts); the least recently used goes first")
+    ap.add_argument("--mixed-graphs", action="store_true", help="replay steps that carry prompt portions from graphs of "
+                    "their padded shapes instead of launching them kernel by kernel: for small models with many live "
+                    "requests, where the host is the bound")
     ap.add_argument("--debug-poison-cache", action="store_true", help="debugging: cache pages hold NaN until written "
                     "and again once given back, so that a read of a key that must not be seen shows")
     args = ap.parse_args(argv)
@@ -57,7 +60,8 @@ def _generate(argv) -> int:
                        memory_fraction=args.memory_fraction, max_context=args.max_context,
                        max_requests=args.max_requests, max_tokens_per_step=args.max_tokens_per_step,
                        prefill_chunk=args.prefill_chunk, admission=args.admission, admit_interval=args.admit_interval, seed=args.seed,
-                       max_graphs=args.max_graphs, debug_poison_cache=args.debug_poison_cache)
+                       max_graphs=args.max_graphs, debug_poison_cache=args.debug_poison_cache,
+                       graph_mixed_steps=args.mixed_graphs)
     if args.model:
         engine = Engine.from_folder(args.model, cfg)
     else:

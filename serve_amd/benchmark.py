@@ -98,6 +98,9 @@ def main(argv=None) -> int:
                          "(serve/run.py:265) beside decode steps of their own")
     ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--admission", choices=["reserve", "optimistic"], default="reserve")
+    ap.add_argument("--mixed-graphs", action="store_true", help="replay steps that carry prompt portions from graphs of "
+                    "their padded shapes instead of launching them kernel by kernel: for small models with many live "
+                    "requests, where the host is the bound")
     ap.add_argument("--phases", action="store_true", help="time the host's phases of the timed run (schedule, "
                     "plan_step, stage_copy, launch, read_back, ...) with named ranges and print their totals; the "
                     "ranges are also roctx markers for `rocprofv3 --marker-trace`")
@@ -110,7 +113,8 @@ def main(argv=None) -> int:
                        max_context=args.max_context, max_requests=args.max_requests,
                        max_tokens_per_step=args.max_tokens_per_step or 2048 + args.max_requests,
                        prefill_chunk=args.prefill_chunk,
-                       admission=args.admission, admit_interval=args.admit_interval, seed=args.seed)
+                       admission=args.admission, admit_interval=args.admit_interval, seed=args.seed,
+                       graph_mixed_steps=args.mixed_graphs)
     print(f"loading {args.model or args.shape} ({args.dtype}) ...", flush=True)
     if args.model:
         engine = Engine.from_folder(args.model, cfg)

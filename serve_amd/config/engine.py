@@ -35,6 +35,13 @@ class EngineConfig:
     device: str = "cuda:0"
     # replay a decode-only step from a captured HIP graph
     use_graphs: bool = True
+    # also capture steps that carry prompt portions beside decoding requests (where steps are launched
+    # ahead of the host), per padded shape.  A step that is launched kernel by kernel costs the host
+    # about 13 us a kernel, which bounds a small model with hundreds of live requests: there the graphs
+    # gain (the reference's workload at the 1B shape with 256 live requests: 67.6k -> 74.8k tokens/s);
+    # where the device is the bound, their padding loses a few percent (3B shape, portions of 512
+    # tokens: 1.45 -> 1.52 s), so they are off unless asked for.
+    graph_mixed_steps: bool = False
     # how many captured steps (one per padded batch size and bucket of contexts) are kept; beyond
     # that the least recently used one is dropped and captured again when its shape comes back
     max_graphs: int = 64

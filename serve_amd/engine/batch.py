@@ -26,6 +26,17 @@ class OutOfPages(RuntimeError):
     """The step needs more pages than are free.  Nothing was allocated."""
 
 
+class _Inert:
+    def __repr__(self):
+        return "INERT"
+
+
+# the request id of a segment that belongs to no request: padding of a step to a fixed shape.  Its
+# tokens are computed like any others but nothing of them is kept: no pages, cache slot -1 (nothing
+# stored), state slot -1, a block table of zeros (it reads whatever page 0 holds).
+INERT = _Inert()
+
+
 @dataclass
 class Segment:
     req_id: object
@@ -116,11 +127,13 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         raise ValueError("a step needs at least one segment")
     seen = set()
     for s in segments:
+        if len(s.tokens) == 0:
+            raise ValueError(f"request {s.req_id!r} brings no tokens")
+        if s.req_id is INERT:
+            continue
         if s.req_id in seen:
             raise ValueError(f"request {s.req_id!r} appears twice in one step")
         seen.add(s.req_id)
-        if len(s.tokens) == 0:
-            raise ValueError(f"request {s.req_id!r} brings no tokens")
         if s.req_id not in cache:
             raise KeyError(f"request {s.req_id!r} is not admitted")
         if len(s.tokens) == 1:
@@ -137,10 +150,14 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
 
     G = cache.num_groups
     ps = cache.page_size
-    before = [cache.tokens_of(s.req_id) for s in segments]
+    inert = [s.req_id is INERT for s in segments]
+    any_inert = any(inert)
+    before = [0 if dead else cache.tokens_of(s.req_id) for s, dead in zip(segments, inert)]
     after = [b + len(s.tokens) for b, s in zip(before, segments)]
     need = [0] * G
-    for s, n in zip(segments, after):
+    for s, n, dead in zip(segments, after, inert):
+        if dead:
+            continue
         if cache.pages_for_tokens(n) > cache.max_pages_per_request:
             raise OutOfPages(f"request {s.req_id!r} would hold {n} tokens, above the context limit of "
                              f"{cache.max_pages_per_request * ps}")
@@ -149,9 +166,10 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
     for g in range(G):
         if need[g] > cache.free_pages(g):
             raise OutOfPages(f"the step needs {need[g]} pages of group {g}, {cache.free_pages(g)} are free")
-    for s, n in zip(segments, after):
-        ok = cache.ensure(s.req_id, n)
-        assert ok
+    for s, n, dead in zip(segments, after, inert):
+        if not dead:
+            ok = cache.ensure(s.req_id, n)
+            assert ok
 
     B_real = len(segments)
     B = max(B_real, pad_segments_to)
@@ -163,7 +181,7 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         MP = fixed_max_pages
     lay = StepLayout(T, B, R, MP, G)
     host = np.zeros(lay.total, dtype=np.int32)
-    if all(len(s.tokens) == 1 for s in segments):
+    if not any_inert and all(len(s.tokens) == 1 for s in segments):
         # one token per request: fill the arrays without a Python loop over requests
         n = B_real
         slots_np = np.fromiter((cache.slot_of(s.req_id) for s in segments), dtype=np.int64, count=n)
@@ -193,14 +211,18 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
     cu_np = np.zeros(n + 1, dtype=np.int64)
     np.cumsum(q_lens, out=cu_np[1:])
     before_np = np.asarray(before, dtype=np.int64)
-    slots_np = np.fromiter((cache.slot_of(s.req_id) for s in segments), dtype=np.int64, count=n)
+    slots_np = np.fromiter((-1 if dead else cache.slot_of(s.req_id) for s, dead in zip(segments, inert)),
+                           dtype=np.int64, count=n)
     host[lay.cu_q: lay.cu_q + n] = cu_np[:n]
     host[lay.ctx_len: lay.ctx_len + n] = after
     host[lay.state_slots: lay.state_slots + n] = slots_np
     host[lay.logit_rows: lay.logit_rows + R] = [int(c) + int(w) for s, c in zip(segments, cu_np) for w in s.want]
+    dead_np = np.asarray(inert, dtype=bool)
     rows_of = []
     for g in range(G):
-        rows = cache.table_rows[g][slots_np]
+        rows = cache.table_rows[g][np.maximum(slots_np, 0)]
+        if any_inert:
+            rows[dead_np] = 0                   # an inert segment reads page 0, whatever it holds
         rows_of.append(rows)
         host[lay.block_tables[g]: lay.block_tables[g] + n * MP].reshape(n, MP)[:] = rows[:, :MP]
     # per token: the single-token segments together, the others one by one
@@ -213,7 +235,7 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         host[lay.positions + at] = b1
         host[lay.seg_of_token + at] = one
         for g in range(G):
-            host[lay.slots[g] + at] = rows_of[g][one, b1 // ps] * ps + b1 % ps
+            host[lay.slots[g] + at] = np.where(dead_np[one], -1, rows_of[g][one, b1 // ps] * ps + b1 % ps)
     for i in np.nonzero(q_np != 1)[0]:
         s, b, a, c0 = segments[i], before[i], after[i], int(cu_np[i])
         m = a - b
@@ -222,7 +244,10 @@ def plan_step(segments: Sequence[Segment], cache: CacheManager, vocab_size: int,
         host[lay.seg_of_token + c0: lay.seg_of_token + c0 + m] = i
         pos = np.arange(b, a)
         for g in range(G):
-            host[lay.slots[g] + c0: lay.slots[g] + c0 + m] = rows_of[g][i, pos // ps] * ps + pos % ps
+            if inert[i]:
+                host[lay.slots[g] + c0: lay.slots[g] + c0 + m] = -1
+            else:
+                host[lay.slots[g] + c0: lay.slots[g] + c0 + m] = rows_of[g][i, pos // ps] * ps + pos % ps
     cu = int(cu_np[n])
     for j in range(pad):           # inert segments: one token, one visible key, nothing stored
         i = B_real + j

@@ -20,30 +20,41 @@ from ..cache.storage import CacheStorage, bytes_per_page, group_windows
 from ..config.engine import EngineConfig
 from ..models.model import Model
 from ..parts.base import Runtime
-from .batch import Segment, StepLayout, context_from, plan_step
+from .batch import INERT, Segment, StepLayout, context_from, plan_step
 
 # padded batch sizes for which decode-only steps are captured into graphs
 GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
 # more rows than that are replayed from graphs only where nobody asks for the logits (steps launched
 # ahead of the host, which sample on the device): such a graph keeps no [rows, vocabulary] buffer
 ASYNC_GRAPH_BATCHES = GRAPH_BATCHES + (384, 512)
+# steps of decoding requests followed by prompt portions, launched ahead of the host, are captured too:
+# the decoding requests padded to one of these counts, the portions (at most MIXED_MAX_PORTIONS with
+# their padding, MIXED_MAX_TOKENS tokens) to a power of two of segments and a multiple of 128 tokens
+MIXED_DECODE_PADS = (8, 32, 64, 128, 256, 384, 512)
+MIXED_MAX_PORTIONS = 32
+MIXED_MAX_TOKENS = 4096
 
 
 class _GraphEntry:
-    """Fixed buffers and the captured graph of decode-only steps of one shape."""
+    """Fixed buffers and the captured graph of steps of one shape: `b_pad` segments of one token each
+    (decode-only steps), or any numbers of tokens, segments and logit rows (steps with prompt portions)."""
 
-    def __init__(self, b_pad: int, max_pages: int, num_groups: int, device: torch.device):
+    def __init__(self, b_pad: int, max_pages: int, num_groups: int, device: torch.device,
+                 tokens: Optional[int] = None, rows: Optional[int] = None):
         self.b_pad = b_pad
-        self.layout = StepLayout(b_pad, b_pad, b_pad, max_pages, num_groups)
-        # after the step's index arrays: where each row's token comes from, and the sampling inputs
+        T = b_pad if tokens is None else tokens
+        R = b_pad if rows is None else rows
+        self.rows = R
+        self.layout = StepLayout(T, b_pad, R, max_pages, num_groups)
+        # after the step's index arrays: where each token comes from, and the sampling inputs of the rows
         o = self.layout.total
         self.off_src_row = o
-        self.off_temps = o + _pad4(b_pad)
-        self.off_keys = o + 2 * _pad4(b_pad)
-        self.total = o + 2 * _pad4(b_pad) + _pad4(2 * b_pad)
+        self.off_temps = o + _pad4(T)
+        self.off_keys = self.off_temps + _pad4(R)
+        self.total = self.off_keys + _pad4(2 * R)
         self.stage = torch.zeros(self.total, dtype=torch.int32).pin_memory()
         self.device_buf = torch.zeros(self.total, dtype=torch.int32, device=device)
-        self.host_tokens = [torch.zeros(b_pad, dtype=torch.int32).pin_memory() for _ in range(2)]
+        self.host_tokens = [torch.zeros(R, dtype=torch.int32).pin_memory() for _ in range(2)]
         self.copied = torch.cuda.Event()
         self.graph = None
         self.keeps_logits = False          # whether the captured step leaves its logits in the runner's buffer
@@ -115,7 +126,8 @@ class ModelRunner:
         # by side), made at the first such step
         self._graph_logits = None
         # tokens sampled by the latest decode launch, by row: the next launch may read them here
-        self.sampled = torch.zeros(max(ASYNC_GRAPH_BATCHES[-1], cfg.max_requests), dtype=torch.int32, device=rt.device)
+        self.sampled = torch.zeros(max(ASYNC_GRAPH_BATCHES[-1], MIXED_DECODE_PADS[-1] + MIXED_MAX_PORTIONS,
+                                       cfg.max_requests), dtype=torch.int32, device=rt.device)
         self._row_of = {}
         self._use_graphs = bool(cfg.use_graphs) and model.graph_safe()
         # steps launched ahead of the host need parts that never read back from the device
@@ -305,6 +317,129 @@ class ModelRunner:
             self.cache.trim(r, n)
         return DecodeHandle(host, ev, len(req_ids))
 
+    # -- steps with prompt portions replayed from graphs ------------------------------------------------
+    def _mixed_shape(self, segments: Sequence[Segment]):
+        """The padded shape under which a step of decoding requests followed by prompt portions is
+        captured, or None if it is run kernel by kernel: (single-token segments in front, padded;
+        segments behind them, padded, at least one of them inert; their tokens, padded to a multiple
+        of 128; buckets of the longest context of either kind)."""
+        if not (self._use_graphs and self.cfg.graph_mixed_steps):
+            return None
+        nd = 0
+        while nd < len(segments) and len(segments[nd].tokens) == 1:
+            nd += 1
+        rest = segments[nd:]
+        if not rest:
+            return None
+        nd_pad = 0 if nd == 0 else next((b for b in MIXED_DECODE_PADS if b >= nd), None)
+        p_tokens = sum(len(s.tokens) for s in rest)
+        n_rest = 1
+        while n_rest < len(rest):
+            n_rest *= 2
+        if (p_tokens + n_rest - len(rest)) % 128:
+            # the padded token count is reached with one more inert segment, of whatever length is missing
+            while n_rest < len(rest) + 1:
+                n_rest *= 2
+        if nd_pad is None or n_rest > MIXED_MAX_PORTIONS:
+            return None
+        p_pad = -(-(p_tokens + n_rest - len(rest)) // 128) * 128
+        longest_d = 1 + max((self.cache.tokens_of(s.req_id) for s in segments[:nd]), default=0)
+        longest_p = max(max(self.cache.tokens_of(s.req_id) + len(s.tokens) for s in rest), p_pad)
+        d_bucket = p_bucket = 256
+        while d_bucket < longest_d:
+            d_bucket *= 2
+        while p_bucket < longest_p:
+            p_bucket *= 2
+        limit = self.cfg.max_pages_per_request * self.cfg.page_size
+        if p_pad > MIXED_MAX_TOKENS or p_pad > limit:         # (the inert portion must fit a block table's row)
+            return None
+        return nd, (nd_pad, n_rest, p_pad, min(d_bucket, limit), min(p_bucket, limit))
+
+    def _launch_mixed_graph(self, req_ids, segments: Sequence[Segment], nd: int, key, src_of_token, temps, keys):
+        """A step of decoding requests and prompt portions, sampled on the device, through the graph of
+        its padded shape.  The padding is made of inert segments: single tokens behind the decoding
+        requests, and behind the prompt portions single tokens and one portion that takes up the rest
+        of the padded token count.  Returns (entry, number of sampled rows, context lengths)."""
+        nd_pad, n_rest, p_pad, d_bucket, p_bucket = key
+        rest = list(segments[nd:])
+        p_tokens = sum(len(s.tokens) for s in rest)
+        # inert single tokens up to the padded number of segments; the last of them takes what is missing of the tokens
+        extra = n_rest - len(rest)
+        filler = p_pad - p_tokens - extra
+        assert (extra > 0 and filler >= 0) or (extra == 0 and filler == 0)
+        padded = (list(segments[:nd]) + [Segment(INERT, [0], []) for _ in range(nd_pad - nd)] + rest
+                  + [Segment(INERT, [0], []) for _ in range(extra - 1)]
+                  + ([Segment(INERT, [0] * (1 + filler), [])] if extra else []))
+        T, B, R = nd_pad + p_pad, nd_pad + n_rest, nd_pad + n_rest
+        mp = min(self.cfg.max_pages_per_request, -(-max(d_bucket, p_bucket) // self.cfg.page_size))
+        with trace.span("plan_step"):
+            lay, host, facts = plan_step(padded, self.cache, self.vocab_size, fixed_max_pages=mp)
+        r_real = lay.R
+        gkey = ("mixed",) + tuple(key)
+        entry = self._graphs.get(gkey)
+        if entry is None:
+            while len(self._graphs) >= max(1, int(self.cfg.max_graphs)):
+                _, old = self._graphs.popitem(last=False)
+                old.copied.synchronize()
+                torch.cuda.current_stream().synchronize()
+                old.graph = None
+            entry = self._graphs[gkey] = _GraphEntry(B, mp, self.cache.num_groups, self.rt.device, tokens=T, rows=R)
+        else:
+            self._graphs.move_to_end(gkey)
+        full = entry.layout
+        with trace.span("stage_copy"):
+            entry.copied.synchronize()
+            sn = entry.stage.numpy()
+            sn[:] = 0
+            # the step's arrays lie as the entry's do, but for the logit rows: the step has fewer
+            for name in ("token_ids", "positions", "seg_of_token", "cu_q", "ctx_len", "state_slots"):
+                a, b = getattr(lay, name), getattr(full, name)
+                n = {"cu_q": B + 1, "ctx_len": B, "state_slots": B}.get(name, T)
+                sn[b: b + n] = host[a: a + n]
+            sn[full.logit_rows: full.logit_rows + r_real] = host[lay.logit_rows: lay.logit_rows + r_real]
+            for g in range(self.cache.num_groups):
+                sn[full.block_tables[g]: full.block_tables[g] + B * mp] = host[lay.block_tables[g]: lay.block_tables[g] + B * mp]
+                sn[full.slots[g]: full.slots[g] + T] = host[lay.slots[g]: lay.slots[g] + T]
+            # where the tokens of the real segments come from: their places among the padded step's tokens
+            src = sn[entry.off_src_row: entry.off_src_row + T]
+            src[:] = -1
+            cu = host[lay.cu_q: lay.cu_q + B]
+            at = {id(s): int(cu[i]) for i, s in enumerate(padded)}
+            for s, row in zip(segments, src_of_token):
+                if row >= 0:
+                    src[at[id(s)]] = row
+            sn[entry.off_temps: entry.off_temps + r_real].view(np.float32)[:] = temps
+            sn[entry.off_keys: entry.off_keys + 2 * r_real].view(np.int64)[:] = keys
+            entry.device_buf.copy_(entry.stage, non_blocking=True)
+            entry.copied.record()
+        with trace.span("launch"):
+            if entry.graph is None:
+                # what the kernels' launches are chosen by, as upper bounds that hold for every step of the shape
+                shape_facts = dict(q_lens=[1] * nd_pad + [p_pad] * n_rest, ctx_lens=[d_bucket] * nd_pad + [p_bucket] * n_rest,
+                                   max_q_len=p_pad, max_ctx_len=max(d_bucket, p_bucket), max_pages=mp, decode_only=False)
+                ctx = context_from(full, entry.device_buf, shape_facts)
+                ctx.src_row = entry.device_buf[entry.off_src_row: entry.off_src_row + T]
+                ctx.prev_tokens = self.sampled
+                t_dev = entry.device_buf[entry.off_temps: entry.off_temps + R].view(torch.float32)
+                k_dev = entry.device_buf[entry.off_keys: entry.off_keys + 2 * R].view(torch.int64)
+
+                def run():
+                    logits = self.model.forward(ctx, self.storage.layers)
+                    ops.sample(logits, t_dev, k_dev, self.sampled[:R])
+                entry.runs += 1
+                run()
+                if entry.runs >= 2:
+                    if self._graph_pool is None:
+                        self._graph_pool = torch.cuda.graph_pool_handle()
+                    g = torch.cuda.CUDAGraph()
+                    torch.cuda.synchronize()
+                    with torch.cuda.graph(g, pool=self._graph_pool):
+                        run()
+                    entry.graph = g
+            else:
+                entry.graph.replay()
+        return entry, r_real, facts["ctx_lens"]
+
     @torch.inference_mode()
     def step_launch(self, req_ids: Sequence, tokens: Sequence[Sequence[Optional[int]]], samples: Sequence[bool],
                     temperatures: Sequence[float], keys: Sequence[int]) -> DecodeHandle:
@@ -319,6 +454,22 @@ class ModelRunner:
                 raise ValueError("only a single token can be left to the device")
             segments = [Segment(r, toks if toks[0] is not None else [0], [len(toks) - 1] if smp else [])
                         for r, toks, smp in zip(req_ids, tokens, samples)]
+            shape = self._mixed_shape(segments)
+            if shape is not None:
+                nd, key = shape
+                src_of_token = [self._row_of[r] if toks[0] is None else -1 for r, toks in zip(req_ids, tokens)]
+                entry, R, _ = self._launch_mixed_graph(req_ids, segments, nd, key, src_of_token,
+                                                       np.asarray(temperatures, dtype=np.float32),
+                                                       np.asarray(keys, dtype=np.int64))
+                self._row_of = {r: i for i, r in enumerate(r for r, smp in zip(req_ids, samples) if smp)}
+                host_tokens = entry.host_tokens[entry.launches & 1]
+                entry.launches += 1
+                host_tokens.copy_(self.sampled[: entry.rows], non_blocking=True)
+                ev = torch.cuda.Event()
+                ev.record()
+                for s in segments:
+                    self.cache.trim(s.req_id, self.cache.tokens_of(s.req_id))
+                return DecodeHandle(host_tokens, ev, R)
             with trace.span("plan_step"):
                 lay, host, facts = plan_step(segments, self.cache, self.vocab_size)
             T, R = lay.T, lay.R

@@ -225,6 +225,44 @@ def test_600_live_requests_step_beyond_the_largest_graph(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["AS", "CS"])
+def test_steps_with_prompt_portions_replayed_from_graphs(tmp_path, name, dtype):
+    """Six slots, portions of eight tokens: most steps are a handful of decoding requests in front of one
+    or two prompt portions, shapes that come again and again, so they are captured (padded with inert
+    segments to 8 decoding requests, 2 or 4 portions and 128 tokens) and replayed; the tokens of every
+    request, greedy or drawn, are the plain model's, and the same as with such graphs switched off."""
+    from serve_amd.engine.engine import Request
+    folder = util.make_folder(tmp_path, name)
+    vocab = util.tiny_config(name).vocab_size
+    rng = random.Random(46)
+    count = 36
+    prompts = [util.random_tokens(rng, rng.randrange(9, 30), vocab) for _ in range(count)]
+    new = [rng.randrange(4, 12) for _ in range(count)]
+    temps = [0.0 if i % 4 else 0.8 for i in range(count)]
+    kw = dict(page_size=8, num_pages=64, max_context=256, max_requests=6, max_tokens_per_step=24, prefill_chunk=8,
+              seed=SEED)
+    engine = make_engine(folder, dtype, graph_mixed_steps=True, **kw)
+    reqs = [Request(torch.tensor(p), len(p), n) for p, n in zip(prompts, new)]
+    log = []
+    out = engine.generate(reqs, temperature=temps, step_log=log)
+    mixed = {k: e for k, e in engine.runner._graphs.items() if k[0] == "mixed"}
+    replayed = [k for k, e in mixed.items() if e.graph is not None and e.launches > 2]
+    assert replayed, f"no step with prompt portions was replayed from a graph; shapes seen: {sorted(mixed)}"
+    assert any(len(s["requests"]) > 2 and max(s["counts"]) > 1 and s["counts"][0] == 1 for s in log)
+    for i, (p, n, r) in enumerate(zip(prompts, new, out)):
+        assert r.error is None and len(r.generated_tokens) == n
+        check_tokens(folder, p, r.generated_tokens.tolist(), dtype, f"{name} {dtype} request {i}", temps[i], i)
+    engine.runner.cache.check_invariants()
+    assert not engine.runner.cache.live_requests() and engine.runner.cache.free_pages(0) == 64
+    # launched kernel by kernel, the same schedule gives the same tokens (float32: to the bit of the argmax)
+    plain_engine = make_engine(folder, dtype, **kw)
+    out2 = plain_engine.generate(reqs, temperature=temps)
+    assert not any(k[0] == "mixed" for k in plain_engine.runner._graphs)
+    if dtype == "float32":
+        assert [r.generated_tokens.tolist() for r in out] == [r.generated_tokens.tolist() for r in out2]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_admission_in_turns_on_the_device(tmp_path, dtype):
     """`admit_interval` 4 with six slots for thirty requests: newcomers start only every fourth step
     while others run, the steps between are decode steps replayed from graphs and launched ahead of

@@ -185,14 +185,14 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
           f"(read + write), reduction {ceil['read'] / 1e12:.2f} TB/s (read), 8192^3 bf16 product "
           f"{ceil['gemm'] / 1e15:.3f} PFLOP/s")
     bw = max(ceil["copy"], ceil["read"], ceil["own_read"], ceil["own_copy"])
-    print(f"{'workload':34s} {'ms/step':>8s} {'tokens/s':>10s} {'GB or TFLOP':>12s} {'achieved':>14s} {'of peak':>8s} "
+    print(f"{'workload':40s} {'ms/step':>8s} {'tokens/s':>10s} {'GB or TFLOP':>12s} {'achieved':>14s} {'of peak':>8s} "
           f"{'of measured':>11s}")
 
     def decode_row(eng, batch, prompt_len, w, n):
         dt, mean_ctx = decode_run(eng, batch, prompt_len, w, n, seed=20 + batch)
         nbytes = weight_bytes(eng.model) + batch * kv_bytes(eng.model, mean_ctx)
         rate = nbytes / (dt / n)
-        print(f"{f'decode, batch {batch}, context ~{int(mean_ctx)}':34s} {dt / n * 1e3:8.3f} {batch * n / dt:10.0f} "
+        print(f"{f'decode, batch {batch}, context ~{int(mean_ctx)}':40s} {dt / n * 1e3:8.3f} {batch * n / dt:10.0f} "
               f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}", flush=True)
     for batch, prompt_len, n in ((1, 256, 250), (8, 256, 250), (64, 256, 250)):
         decode_row(engine, batch, prompt_len, 4, n)
@@ -200,7 +200,7 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
     T = 2048
     pt = prefill_run(engine, T, repeats=5, seed=7)
     fl = prefill_flops(engine.model, T)
-    print(f"{'prefill, 2,048 tokens':34s} {pt * 1e3:8.3f} {T / pt:10.0f} {fl / 1e12:6.3f} TFLOP {fl / pt / 1e15:7.3f} PFLOP/s "
+    print(f"{'prefill, 2,048 tokens':40s} {pt * 1e3:8.3f} {T / pt:10.0f} {fl / 1e12:6.3f} TFLOP {fl / pt / 1e15:7.3f} PFLOP/s "
           f"{fl / pt / BF16_PEAK:8.3f} {fl / pt / ceil['gemm']:11.3f}", flush=True)
     if make_engine is not None:
         del engine
@@ -216,7 +216,7 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
         dt, mean_ctx = decode_run(eng, 8, 4096 - 64 - 16 - 3 - head_start(eng, 8, 4096), 16, 64, seed=28)
         nbytes = weight_bytes(eng.model, 4) + 8 * kv_bytes(eng.model, mean_ctx, 4)
         rate = nbytes / (dt / 64)
-        print(f"{f'float32 decode, batch 8, context ~{int(mean_ctx)}':34s} {dt / 64 * 1e3:8.3f} {8 * 64 / dt:10.0f} "
+        print(f"{f'float32 decode, batch 8, context ~{int(mean_ctx)}':40s} {dt / 64 * 1e3:8.3f} {8 * 64 / dt:10.0f} "
               f"{nbytes / 1e9:9.3f} GB {rate / 1e12:9.2f} TB/s {rate / HBM_PEAK:8.3f} {rate / bw:11.3f}", flush=True)
     return 0
 

@@ -177,7 +177,42 @@ class ModelRunner:
             self.cache.trim(s.req_id, n)
         return logits
 
-    # -- decode-only steps replayed from HIP graphs ---------------------------------------------------
+    # -- steps replayed from HIP graphs ---------------------------------------------------------------
+    def _graph_entry(self, key, make):
+        """The entry of a captured shape, made by `make()` if it is new; the most recently used
+        entries are kept, up to cfg.max_graphs."""
+        entry = self._graphs.get(key)
+        if entry is not None:
+            self._graphs.move_to_end(key)
+            return entry
+        while len(self._graphs) >= max(1, int(self.cfg.max_graphs)):
+            # the least recently used shape goes: its graph, index buffers and pinned staging memory
+            # (a copy out of that memory may still run: wait for it)
+            _, old = self._graphs.popitem(last=False)
+            old.copied.synchronize()
+            torch.cuda.current_stream().synchronize()
+            old.graph = None
+        entry = self._graphs[key] = make()
+        return entry
+
+    def _run_then_capture(self, entry, run):
+        """Run a shape's step kernel by kernel; from its second run on (every library is loaded and
+        warm by then) also capture it for the steps that follow.  All graphs take their intermediate
+        buffers from one pool (they never run side by side), and none keeps memory of its own beyond
+        its index buffers."""
+        entry.runs += 1
+        result = run()
+        if entry.runs >= 2:
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            g = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g, pool=self._graph_pool):
+                run()
+            entry.graph = g
+        return result
+
+    # -- decode-only steps ------------------------------------------------------------------------------
     def _decode_core(self, segments: Sequence[Segment], temps=None, keys=None, src_rows=None, keep_logits=True):
         """One token per request, sampling included.  The kernel sequence of such a step depends
         only on the padded batch size and on the bucket of the longest context (which fixes the
@@ -200,19 +235,8 @@ class ModelRunner:
         with trace.span("plan_step"):
             lay, host, facts = plan_step(segments, self.cache, self.vocab_size, pad_segments_to=b_pad,
                                          fixed_max_pages=mp)
-        key = (b_pad, bucket)
-        entry = self._graphs.get(key)
-        if entry is None:
-            while len(self._graphs) >= max(1, int(self.cfg.max_graphs)):
-                # the least recently used shape goes: its graph, index buffers and pinned staging memory
-                # (a copy out of that memory may still run: wait for it)
-                _, old = self._graphs.popitem(last=False)
-                old.copied.synchronize()
-                torch.cuda.current_stream().synchronize()
-                old.graph = None
-            entry = self._graphs[key] = _GraphEntry(b_pad, mp, self.cache.num_groups, self.rt.device)
-        else:
-            self._graphs.move_to_end(key)
+        entry = self._graph_entry((b_pad, bucket),
+                                  lambda: _GraphEntry(b_pad, mp, self.cache.num_groups, self.rt.device))
         full = entry.layout
         with trace.span("stage_copy"):
             entry.copied.synchronize()          # the previous step's copy out of the staging buffer is done
@@ -260,20 +284,8 @@ class ModelRunner:
                         # a head that does not write where it is told (a part that knows no `out`)
                         self._graph_logits[:b_pad].copy_(logits)
                     return self._graph_logits[:b_pad]
-                entry.runs += 1
-                logits = run()
-                if entry.runs >= 2:
-                    # every library is loaded and warm by now: capture for the following steps
-                    # all graphs take their intermediate buffers from one pool (they never run side by
-                    # side), and none keeps memory of its own beyond its index buffers
-                    if self._graph_pool is None:
-                        self._graph_pool = torch.cuda.graph_pool_handle()
-                    g = torch.cuda.CUDAGraph()
-                    torch.cuda.synchronize()
-                    with torch.cuda.graph(g, pool=self._graph_pool):
-                        run()
-                    entry.graph = g
-                    entry.keeps_logits = shared
+                logits = self._run_then_capture(entry, run)
+                entry.keeps_logits = shared
             else:
                 entry.graph.replay()
                 logits = self._graph_logits[:b_pad] if entry.keeps_logits else None
@@ -375,17 +387,8 @@ class ModelRunner:
         with trace.span("plan_step"):
             lay, host, facts = plan_step(padded, self.cache, self.vocab_size, fixed_max_pages=mp)
         r_real = lay.R
-        gkey = ("mixed",) + tuple(key)
-        entry = self._graphs.get(gkey)
-        if entry is None:
-            while len(self._graphs) >= max(1, int(self.cfg.max_graphs)):
-                _, old = self._graphs.popitem(last=False)
-                old.copied.synchronize()
-                torch.cuda.current_stream().synchronize()
-                old.graph = None
-            entry = self._graphs[gkey] = _GraphEntry(B, mp, self.cache.num_groups, self.rt.device, tokens=T, rows=R)
-        else:
-            self._graphs.move_to_end(gkey)
+        entry = self._graph_entry(("mixed",) + tuple(key),
+                                  lambda: _GraphEntry(B, mp, self.cache.num_groups, self.rt.device, tokens=T, rows=R))
         full = entry.layout
         with trace.span("stage_copy"):
             entry.copied.synchronize()
@@ -426,16 +429,7 @@ class ModelRunner:
                 def run():
                     logits = self.model.forward(ctx, self.storage.layers)
                     ops.sample(logits, t_dev, k_dev, self.sampled[:R])
-                entry.runs += 1
-                run()
-                if entry.runs >= 2:
-                    if self._graph_pool is None:
-                        self._graph_pool = torch.cuda.graph_pool_handle()
-                    g = torch.cuda.CUDAGraph()
-                    torch.cuda.synchronize()
-                    with torch.cuda.graph(g, pool=self._graph_pool):
-                        run()
-                    entry.graph = g
+                self._run_then_capture(entry, run)
             else:
                 entry.graph.replay()
         return entry, r_real, facts["ctx_lens"]

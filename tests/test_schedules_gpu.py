@@ -375,6 +375,59 @@ def test_poisoned_cache_changes_nothing(tmp_path, dtype):
     assert torch.isnan(engine.runner.storage.layers[1].v_pages).all()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_models_requests_and_settings_through_the_scheduler(tmp_path, seed):
+    """A random configuration (head sizes 16 to 128, one to three KV heads, groups of one to five,
+    widths and vocabularies that are no power of two), random requests and four random settings of
+    the engine (dtype, page size, so few pages that requests wait or are preempted, either admission,
+    token budgets down to 64, portions down to 16, graphs, graphs of mixed steps, the poisoned cache,
+    admission in turns): every greedy token must be a best token of the plain model within the
+    dtype's error, and every page comes back."""
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.llama import Llama3RopeScaling, LlamaConfig
+    from serve_amd.engine.engine import Engine, Request
+    from serve_amd.weights.loader import write_random_model
+    rng = random.Random(1000 + seed)
+    kv_heads, group = rng.choice([1, 2, 3]), rng.choice([1, 2, 4, 5])
+    cfg = LlamaConfig(vocab_size=rng.randrange(50, 900), hidden_size=rng.choice([64, 72, 136, 256]),
+                      intermediate_size=8 * rng.randrange(8, 40), num_hidden_layers=rng.choice([1, 2, 3]),
+                      num_attention_heads=kv_heads * group, num_key_value_heads=kv_heads,
+                      head_dim=rng.choice([16, 32, 64, 80, 128]), rms_norm_eps=rng.choice([1e-5, 1e-6]),
+                      rope_theta=rng.choice([10000.0, 500000.0]),
+                      rope_scaling=rng.choice([None, Llama3RopeScaling(8.0, 1.0, 4.0, 64)]),
+                      tie_word_embeddings=rng.choice([True, False]))
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=seed, dtype=torch.bfloat16, scales=util.SHARP_SCALES)
+    w, pc = util.plain_weights(folder), util.plain_config(folder)
+    count = rng.randrange(8, 32)
+    prompts = [util.random_tokens(rng, rng.choice([1, 2, 5, 17, 40, 90, 150, 260]), cfg.vocab_size) for _ in range(count)]
+    news = [rng.choice([1, 2, 7, 20, 45]) for _ in range(count)]
+    # the plain model's logits after every token of a request depend on the engine's tokens: teacher-forced below
+    for trial in range(4):
+        dtype = rng.choice(DTYPES)
+        ps = rng.choice([4, 8, 16, 32])
+        need = max(-(-(len(p) + n) // ps) for p, n in zip(prompts, news))
+        settings = dict(dtype=dtype, page_size=ps, max_context=512, max_requests=rng.choice([3, 8, 16, 64]),
+                        num_pages=rng.choice([need + 1, 2 * need, 8 * need, 4096]),
+                        admission=rng.choice(["reserve", "optimistic"]),
+                        max_tokens_per_step=rng.choice([64, 200, 2048]), prefill_chunk=rng.choice([16, 50, 128, 2048]),
+                        graph_mixed_steps=rng.choice([True, False]), debug_poison_cache=rng.choice([True, False]),
+                        use_graphs=rng.choice([True, True, False]), admit_interval=rng.choice([1, 1, 3]))
+        eng = Engine.from_folder(folder, EngineConfig(**settings))
+        out = eng.generate([Request(torch.tensor(p), len(p), n) for p, n in zip(prompts, news)], temperature=0.0)
+        eng.runner.cache.check_invariants()
+        assert not eng.runner.cache.live_requests()
+        assert eng.runner.cache.free_pages() == settings["num_pages"]
+        tol = 2e-2 if dtype == "bfloat16" else 1e-4
+        for i, (p, n, r) in enumerate(zip(prompts, news, out)):
+            assert r.error is None, (settings, r.error)
+            got = r.generated_tokens.tolist()
+            assert len(got) == n
+            logits = llama_plain.forward(p + got[:-1], w, pc)[len(p) - 1:]
+            gap = logits.max(dim=-1).values - logits[torch.arange(n), torch.tensor(got)]
+            assert gap.max().item() <= tol, (settings, i, gap.argmax().item(), gap.max().item())
+        del eng
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_stop_tokens_end_a_request_and_free_its_pages(tmp_path, dtype):
     """A token id that the greedy continuation of request 1 contains ends it there (the id stays

@@ -1,6 +1,8 @@
 // bf16 matrix products on the matrix cores for few rows of activations (decode steps and short
 // prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
-// Two kernels: gemm_skinny_kernel for one or two rows, gemm_mid_kernel for up to 64 (per pass).
+// Three kernels: gemm_skinny_kernel for one or two rows, gemm_mid_kernel for up to 128 (per pass),
+// and gemm_wide_kernel, which brings both operands into LDS without passing registers and takes
+// the products of 17 to 128 rows where that is faster (see pick_wide).
 //
 // The work is bound by reading W.  In the first, a wave owns RT tiles of 16 rows of W and walks a
 // slice of K in steps of 32; the KS waves of a workgroup split K between them and add their partial sums
@@ -512,6 +514,233 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
   return 0;
 }
 
+// The same products with both operands loaded straight into LDS (global_load_lds: 16 bytes a lane,
+// no registers in between, so nothing has to be held for stages that are on their way).  A
+// workgroup owns 64 rows of W (four tiles of 16) and BM = 64 MW rows of A; a stage is 64 columns
+// of K of both, one kilobyte an instruction (8 rows of 128 bytes), in a ring of NB stages.  A row
+// of a stage holds 8 segments of 16 bytes; segment s of row r lies at slot s ^ ((r >> 1) & 7), so
+// that the 16 lanes of a fragment read (16 rows, one segment) touch every bank once; the loads
+// apply the same exchange on their way in by choosing which segment a lane fetches.  Eight waves:
+// wave = (mw, kh), mw = which quarter of the rows (MW tiles of 16), kh = which half (32 columns)
+// of every stage; the two halves add their sums through LDS at the end, in a fixed order.  A
+// wave waits for its own loads with the counter of loads in flight (they land in order), then
+// the workgroup's barrier says that everybody's have landed and that the stage before has been
+// read, so its place in the ring can be filled again.  Needs K to be whole stages for every part
+// (K % (64 parts) == 0: a stage cannot be zeroed on its way into LDS); rows beyond M and N are
+// read from the last row and their sums never stored.
+#define SA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
+
+template <int MW, int NB, typename TC, int EPI>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                       TC* __restrict__ C, int M, int N, int K, int up_offset) {
+  constexpr bool SWIGLU = EPI == EPI_SWIGLU;
+  static_assert(EPI == EPI_PLAIN || EPI == EPI_SWIGLU, "the rotating epilogue stays with gemm_mid_kernel");
+  constexpr int NT = 4;                            // tiles of 16 weight rows; SwiGLU: two of the gate, two of up
+  constexpr int BM = 64 * MW;
+  constexpr int BN = 16 * NT;
+  constexpr int A_BYTES = BM * 128;
+  constexpr int STAGE_BYTES = A_BYTES + BN * 128;
+  constexpr int COLS = SWIGLU ? BN / 2 : BN;       // output columns of a workgroup
+  constexpr int ND = MW + 1;                       // loads per wave and stage: MW of A, one of W
+  static_assert(ND * (NB - 1) < 64, "the counter of loads in flight has six bits");
+  static_assert(NB * STAGE_BYTES >= 4 * MW * NT * 4 * 64 * 4, "the sums of the second K half reuse the ring");
+  extern __shared__ __attribute__((aligned(16))) u32x4_t wide_lds[];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int mw = wave & 3;
+  const int kh = wave >> 2;
+  const int m0 = blockIdx.z * BM;
+  const int n0 = blockIdx.x * COLS;
+
+  const int nstages = (K >> 6) / gridDim.y;
+  const int k_begin = blockIdx.y * nstages * 64;
+  // (stages walked in an order rotated per workgroup, as in gemm_mid_kernel; it depends on the
+  // weight rows only)
+  const int rot = (int)(blockIdx.x % (unsigned)nstages);
+  auto stage_k = [&](int s) __attribute__((always_inline)) {
+    int t = min(s, nstages - 1) + rot;             // past the last stage: the last again (nobody reads it)
+    if (t >= nstages) t -= nstages;
+    return k_begin + t * 64;
+  };
+  C += (size_t)blockIdx.y * M * N;
+
+  // what this lane fetches: instruction d of wave w fills rows 8 (w MW + d) .. + 7 of the stage's
+  // activations, 8 lanes a row; the wave's last instruction fills 8 of the 64 weight rows
+  const bf16_t* src[ND];
+#pragma unroll
+  for (int d = 0; d < MW; ++d) {
+    const int row = (wave * MW + d) * 8 + (lane >> 3);
+    const int seg = (lane & 7) ^ ((row >> 1) & 7);
+    src[d] = A + (size_t)min(m0 + row, M - 1) * K + seg * 8;
+  }
+  {
+    const int row = wave * 8 + (lane >> 3);
+    const int seg = (lane & 7) ^ ((row >> 1) & 7);
+    int n;
+    if (SWIGLU) n = row < BN / 2 ? min(n0 + row, N - 1) : up_offset + min(n0 + row - BN / 2, N - 1);
+    else n = min(n0 + row, N - 1);
+    src[MW] = W + (size_t)n * K + seg * 8;
+  }
+  typedef __attribute__((address_space(3))) u32x4_t* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  const lds_ptr_t lds0 = (lds_ptr_t)wide_lds;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds0;
+  // this lane's fragment of tile 0 of its rows (and of weight tile 0), in the first place of the ring
+  const uint32_t slot16 = (uint32_t)(((kh * 4 + g) ^ ((c >> 1) & 7)) * 16);
+  const uint32_t a_addr = lds_base + (uint32_t)((mw * MW * 16 + c) * 128) + slot16;
+  const uint32_t w_addr = lds_base + A_BYTES + (uint32_t)(c * 128) + slot16;
+
+  floatx4_t acc[MW][NT];
+#pragma unroll
+  for (int mt = 0; mt < MW; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+  auto fetch = [&](int s) __attribute__((always_inline)) {
+    const int k0 = stage_k(s);
+    const lds_ptr_t buf = lds0 + (s % NB) * (STAGE_BYTES / 16);
+#pragma unroll
+    for (int d = 0; d < MW; ++d)
+      __builtin_amdgcn_global_load_lds((gptr_t)(src[d] + k0), (__attribute__((address_space(3))) void*)
+                                       (buf + (wave * MW + d) * 64), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)(src[MW] + k0), (__attribute__((address_space(3))) void*)
+                                     (buf + A_BYTES / 16 + wave * 64), 16, 0, 0);
+  };
+
+#pragma unroll
+  for (int i = 0; i < NB - 1; ++i) fetch(i);
+  for (int s = 0; s < nstages; ++s) {
+    SA_WAIT_VMCNT(ND * (NB - 2));              // this wave's part of stage s lies in LDS
+    __builtin_amdgcn_s_barrier();              // everybody's does, and everybody has read stage s - 1
+    fetch(s + NB - 1);
+    const uint32_t boff = (uint32_t)((s % NB) * STAGE_BYTES);
+    // (the reads are written as instructions of their own: the compiler does not see the loads
+    // into LDS as stores, and would otherwise wait for all of them before every read)
+    Frag af[MW], wf[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wf[nt].r) : "v"(w_addr + boff), "n"(nt * 16 * 128));
+#pragma unroll
+    for (int mt = 0; mt < MW; ++mt)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[mt].r) : "v"(a_addr + boff), "n"(mt * 16 * 128));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) asm volatile("" : "+v"(wf[nt].r));
+#pragma unroll
+    for (int mt = 0; mt < MW; ++mt) asm volatile("" : "+v"(af[mt].r));
+#pragma unroll
+    for (int mt = 0; mt < MW; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt].v, af[mt].v, acc[mt][nt], 0, 0, 0);
+  }
+
+  // the second half of K hands its sums over through LDS (no load into LDS may still be on its way)
+  float* red = reinterpret_cast<float*>(wide_lds);
+  SA_WAIT_VMCNT(0);
+  __syncthreads();
+  if (kh == 1) {
+#pragma unroll
+    for (int mt = 0; mt < MW; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        *reinterpret_cast<floatx4_t*>(&red[((((mw * MW + mt) * NT + nt) * 64) + lane) * 4]) = acc[mt][nt];
+  }
+  __syncthreads();
+  if (kh == 1) return;
+#pragma unroll
+  for (int mt = 0; mt < MW; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      acc[mt][nt] += *reinterpret_cast<const floatx4_t*>(&red[((((mw * MW + mt) * NT + nt) * 64) + lane) * 4]);
+
+  // lane l holds C[m = row tile's row l % 16][n = 4 (l / 16) .. + 3] of every tile pair
+#pragma unroll
+  for (int mt = 0; mt < MW; ++mt) {
+    const int m = m0 + (mw * MW + mt) * 16 + c;
+    if (m >= M) continue;
+#pragma unroll
+    for (int nt = 0; nt < (SWIGLU ? NT / 2 : NT); ++nt) {
+      const int n = n0 + nt * 16 + 4 * g;
+      float o[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (SWIGLU) {
+          const float gt = acc[mt][nt][r];
+          o[r] = (gt / (1.f + __expf(-gt))) * acc[mt][SWIGLU ? nt + NT / 2 : nt][r];
+        } else {
+          o[r] = acc[mt][nt][r];
+        }
+      }
+      if (n + 3 < N) {
+        store4(C + (size_t)m * N + n, o, (N & 3) == 0);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) C[(size_t)m * N + n + r] = from_float<TC>(o[r]);
+      }
+    }
+  }
+}
+
+template <int MW, int NB, typename TC, int EPI>
+static int launch_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
+                       hipStream_t stream) {
+  constexpr int BM = 64 * MW;
+  constexpr int COLS = EPI == EPI_SWIGLU ? 32 : 64;
+  constexpr size_t lds_bytes = (size_t)NB * (BM * 128 + 64 * 128);
+  static_assert(lds_bytes <= 160 * 1024, "the LDS of a compute unit");
+  dim3 grid((N + COLS - 1) / COLS, parts, (M + BM - 1) / BM);
+  if (grid.z > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
+  auto kernel = gemm_wide_kernel<MW, NB, TC, EPI>;
+  static bool allowed[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SA_ERR_ARG;
+  if (!allowed[dev]) {        // more dynamic LDS than a kernel gets without asking
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    allowed[dev] = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, stream, (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K,
+                     up_offset);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// Which products gemm_wide_kernel takes, from timings beside gemm_mid_kernel at the sizes of the
+// Llama-3 family with cold weights, 16 to 256 rows (in microseconds, wide against mid):
+//   gate/up + SwiGLU, K 2048, 2 x 8192 rows of W: 13.8 / 17.0 at 32 rows, 15.4 / 19.3 at 64, 18.7 / 26.1 at 128;
+//     K 4096, 2 x 14336: level up to 64 rows, 66 / 73 at 80, 73 / 82 at 128;
+//   down_proj in fp32 parts, K 8192: 9.6 / 10.0 at 32, 10.9 / 13.1 at 64, 15.0 / 17.6 at 128 (eight parts
+//     against four); K 14336: 24 / 28 at 32, 27 / 34 at 64, 43 / 52 at 128;
+//   o_proj, K 2048: 6.7 / 6.1 at 64, 9.6 / 8.5 at 128 (mid stays); K 4096: 10.9 / 12.3 at 64, 14.9 / 17.4 at 128;
+//   the head over 128,256 rows of W, K 2048: 116 / 111 at 32, 128 / 132 at 64, 154 / 165 at 96, 168 / 190 at 128;
+//     K 4096: 188 / 298 at 16, 223 / 301 at 64, 286 / 330 at 128.
+// At 16 rows and fewer gemm_mid_kernel is level or ahead everywhere but for that last matrix.
+template <typename TC, int EPI>
+static bool takes_wide(int M, int N, int K, int parts) {
+  if (EPI == EPI_QKV_ROPE || M > 128 || (K & 63) || parts < 1 || (K >> 6) % parts || (K >> 6) / parts < 2) return false;
+  if (EPI == EPI_SWIGLU) return M > 16;
+  if (N >= 8192) return parts == 1 && (M >= 48 || (K >= 4096 && M > 8));       // the head
+  // narrow matrices with a long K, cut into enough parts to give half the compute units a workgroup
+  return M > 16 && K >= 4096 && ((N + 63) / 64) * parts >= 128;
+}
+
+template <typename TC, int EPI>
+static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
+                     hipStream_t stream) {
+  // one or two groups of 64 rows; the ring as deep as LDS allows up to five stages
+  if constexpr (EPI != EPI_QKV_ROPE) {
+    if (M <= 64) return launch_wide<1, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+    return launch_wide<2, 5, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+  }
+  return SA_ERR_ARG;
+}
+
 // up to this many rows take gemm_skinny_kernel, more take gemm_mid_kernel
 // Which kernel and which workgroup shape a product takes, from a sweep over both kernels and their
 // shapes at the sizes of the Llama-3 family (widths 2048 to 4096), 1 to 64 rows, weights cold.
@@ -633,6 +862,14 @@ static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int 
   return SA_ERR_ARG;
 }
 
+// whether a product of these sizes goes to gemm_wide_kernel (epi: EPI_PLAIN or EPI_SWIGLU, for which N
+// is the number of gate rows): for the caller's choice of `parts`, and for tests
+extern "C" int sa_gemm_bf16_takes_wide(int epi, int M, int N, int K, int parts) {
+  if (epi == EPI_SWIGLU) return takes_wide<bf16_t, EPI_SWIGLU>(M, N, K, parts) ? 1 : 0;
+  if (epi == EPI_PLAIN) return takes_wide<float, EPI_PLAIN>(M, N, K, parts) ? 1 : 0;
+  return 0;
+}
+
 // C = A W^T; c_dtype SA_BF16 or SA_F32.  parts > 1 (fp32 only): C is [parts, M, N] and holds
 // partial sums over `parts` slices of K, to be added by the consumer.
 extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K,
@@ -641,8 +878,13 @@ extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_
   if (K <= 0 || (K & 7) || parts < 1) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
   if (!takes_skinny<float, EPI_PLAIN>(M, N, none)) {
-    if (c_dtype == SA_BF16 && parts == 1) return pick_mid<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
-    if (c_dtype == SA_F32) return pick_mid<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
+    const bool wide = takes_wide<float, EPI_PLAIN>(M, N, K, parts);
+    if (c_dtype == SA_BF16 && parts == 1)
+      return wide ? pick_wide<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, stream)
+                  : pick_mid<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
+    if (c_dtype == SA_F32)
+      return wide ? pick_wide<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, stream)
+                  : pick_mid<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
     return SA_ERR_UNSUPPORTED;
   }
   if (c_dtype == SA_BF16 && parts == 1) return pick_skinny<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
@@ -656,6 +898,7 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
   if (M <= 0 || I <= 0) return 0;
   if (K <= 0 || (K & 7)) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
+  if (takes_wide<bf16_t, EPI_SWIGLU>(M, I, K, 1)) return pick_wide<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, stream);
   if (!takes_skinny<bf16_t, EPI_SWIGLU>(M, I, none)) return pick_mid<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   return pick_skinny<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
 }

@@ -463,6 +463,13 @@ def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tor
     return out
 
 
+def gemm_takes_wide(M: int, N: int, K: int, parts: int = 1, swiglu: bool = False) -> bool:
+    """Whether the few-row product of these sizes runs as the kernel that keeps both operands in LDS
+    (for SwiGLU, N is the number of gate rows)."""
+    lib = load_library("gemm_mfma")
+    return bool(lib.sa_gemm_bf16_takes_wide(c_int(1 if swiglu else 0), c_int(M), c_int(N), c_int(K), c_int(parts)))
+
+
 def split_k_parts(M: int, N: int, K: int) -> int:
     """Into how many slices the inner dimension of a few-row product is cut across workgroups so
     that a matrix with few rows still fills the chip: 1 means no cut.  One or two rows: a workgroup
@@ -472,6 +479,15 @@ def split_k_parts(M: int, N: int, K: int) -> int:
         return 1
     cus = compute_units()
     parts = 1
+    if 16 < M <= SKINNY_MAX_ROWS and K >= 4096 and K % 64 == 0:
+        # the kernel with both operands in LDS takes these (csrc/gemm_mfma.hip, takes_wide): 64 weight
+        # rows a workgroup, whole stages of 64 columns for every part
+        groups = -(-N // 64)
+        while parts < 8 and groups * parts < cus and K // (parts * 2) >= 512:
+            parts *= 2
+        if (K // 64) % parts == 0 and groups * parts >= 128:
+            return parts
+        parts = 1
     if M > 2:
         groups = -(-N // 32)
         while parts < 8 and groups * parts < cus and K // (parts * 2) >= 512:

@@ -626,6 +626,50 @@ def test_swiglu_bf16(M, I, K):
     torch.testing.assert_close(out2.double(), want, atol=3e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("kind,M,N,K,parts", [
+    # gate/up with SwiGLU: 17 to 128 rows, K whole stages of 64; widths that are no multiple of a workgroup's 32
+    ("swiglu", 17, 40, 128, 1), ("swiglu", 33, 1000, 192, 1), ("swiglu", 64, 8192, 2048, 1),
+    ("swiglu", 100, 77, 256, 1), ("swiglu", 128, 8200, 320, 1), ("swiglu", 65, 12300, 4096, 1),
+    # the head: many rows of W, 48 rows and more (9 and more with a long K)
+    ("plain", 48, 8200, 128, 1), ("plain", 64, 32064, 192, 1), ("plain", 100, 9001, 192, 1), ("plain", 9, 8200, 4096, 1),
+    ("plain", 128, 8195, 2048, 1),
+    # narrow matrices with a long K, in parts
+    ("parts", 32, 2048, 8192, 8), ("parts", 64, 4096, 4096, 4), ("parts", 70, 1664, 4480, 5), ("parts", 128, 2050, 8192, 8),
+    ("parts", 17, 4100, 14336, 2)])
+def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
+    """The sizes that `gemm_wide_kernel` takes (asserted), against the float64 product: row counts that are no
+    multiple of 16, widths that are no multiple of a workgroup's columns, one or two groups of 64 rows, parts."""
+    from serve_amd import ops
+    assert ops.gemm_takes_wide(M, N, K, parts, swiglu=kind == "swiglu")
+    a = rnd((M, K), torch.bfloat16, 14)
+    if kind == "swiglu":
+        w = rnd((2 * N, K), torch.bfloat16, 15, 0.05)
+        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.swiglu_bf16(a, w, out)
+        gu = a.double() @ w.double().T
+        want = torch.nn.functional.silu(gu[:, :N]) * gu[:, N:]
+        torch.testing.assert_close(out.double(), want, atol=2e-2, rtol=1e-2)
+        return
+    w = rnd((N, K), torch.bfloat16, 15, 0.05)
+    want = a.double() @ w.double().T
+    if kind == "plain":
+        for dt, t in ((torch.float32, dict(atol=2e-4 * K ** 0.5, rtol=1e-4)), (torch.bfloat16, dict(atol=3e-2, rtol=1e-2))):
+            out = torch.full((M, N), float("nan"), dtype=dt, device=DEV)
+            ops.gemm_bf16_skinny(a, w, out)
+            torch.testing.assert_close(out.double(), want, **t)
+    else:
+        out = torch.full((parts, M, N), float("nan"), dtype=torch.float32, device=DEV)
+        ops.gemm_bf16_skinny(a, w, out)
+        torch.testing.assert_close(out.double().sum(0), want, atol=2e-4 * K ** 0.5, rtol=1e-4)
+        assert not torch.allclose(out[0].double(), want)       # really parts
+        if N >= 2048:
+            # the number of parts that the linear part chooses for such a matrix is one this kernel takes
+            assert ops.gemm_takes_wide(M, N, K, ops.split_k_parts(M, N, K))
+    # rows beyond these sizes and inner sizes that are no whole stages stay with the other kernels
+    assert not ops.gemm_takes_wide(16, N, K, parts, swiglu=kind == "swiglu") or kind == "plain"
+    assert not ops.gemm_takes_wide(129, N, K, parts) and not ops.gemm_takes_wide(M, N, K + 8, parts)
+
+
 def test_kernels_refuse_what_they_do_not_take():
     from serve_amd import ops
     a = rnd((4, 12), torch.bfloat16, 1)

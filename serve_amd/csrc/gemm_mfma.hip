@@ -516,8 +516,9 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
 
 // The same products with both operands loaded straight into LDS (global_load_lds: 16 bytes a lane,
 // no registers in between, so nothing has to be held for stages that are on their way).  A
-// workgroup owns 64 rows of W (four tiles of 16) and BM = 64 MW rows of A; a stage is 64 columns
-// of K of both, one kilobyte an instruction (8 rows of 128 bytes), in a ring of NB stages.  A row
+// workgroup owns NT tiles of 16 rows of W (four, or eight for matrices with so many rows that four
+// would give more workgroups than one round of the chip holds) and BM = 64 MW rows of A; a stage is 64
+// columns of K of both, one kilobyte an instruction (8 rows of 128 bytes), in a ring of NB stages.  A row
 // of a stage holds 8 segments of 16 bytes; segment s of row r lies at slot s ^ ((r >> 1) & 7), so
 // that the 16 lanes of a fragment read (16 rows, one segment) touch every bank once; the loads
 // apply the same exchange on their way in by choosing which segment a lane fetches.  Eight waves:
@@ -530,18 +531,19 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
 // read from the last row and their sums never stored.
 #define SA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
 
-template <int MW, int NB, typename TC, int EPI>
+template <int MW, int NT, int NB, typename TC, int EPI>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                        TC* __restrict__ C, int M, int N, int K, int up_offset) {
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
   static_assert(EPI == EPI_PLAIN || EPI == EPI_SWIGLU, "the rotating epilogue stays with gemm_mid_kernel");
-  constexpr int NT = 4;                            // tiles of 16 weight rows; SwiGLU: two of the gate, two of up
+  static_assert(NT == 4 || NT == 8, "tiles of 16 weight rows, 8 rows a wave and instruction; SwiGLU: half of the gate, half of up");
   constexpr int BM = 64 * MW;
   constexpr int BN = 16 * NT;
   constexpr int A_BYTES = BM * 128;
   constexpr int STAGE_BYTES = A_BYTES + BN * 128;
   constexpr int COLS = SWIGLU ? BN / 2 : BN;       // output columns of a workgroup
-  constexpr int ND = MW + 1;                       // loads per wave and stage: MW of A, one of W
+  constexpr int NWI = NT / 4;                      // weight loads per wave and stage
+  constexpr int ND = MW + NWI;                     // loads per wave and stage
   static_assert(ND * (NB - 1) < 64, "the counter of loads in flight has six bits");
   static_assert(NB * STAGE_BYTES >= 4 * MW * NT * 4 * 64 * 4, "the sums of the second K half reuse the ring");
   extern __shared__ __attribute__((aligned(16))) u32x4_t wide_lds[];
@@ -568,7 +570,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   C += (size_t)blockIdx.y * M * N;
 
   // what this lane fetches: instruction d of wave w fills rows 8 (w MW + d) .. + 7 of the stage's
-  // activations, 8 lanes a row; the wave's last instruction fills 8 of the 64 weight rows
+  // activations, 8 lanes a row; the wave's last instructions fill 8 weight rows each
   const bf16_t* src[ND];
 #pragma unroll
   for (int d = 0; d < MW; ++d) {
@@ -576,13 +578,14 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
     const int seg = (lane & 7) ^ ((row >> 1) & 7);
     src[d] = A + (size_t)min(m0 + row, M - 1) * K + seg * 8;
   }
-  {
-    const int row = wave * 8 + (lane >> 3);
+#pragma unroll
+  for (int d = 0; d < NWI; ++d) {
+    const int row = (wave * NWI + d) * 8 + (lane >> 3);
     const int seg = (lane & 7) ^ ((row >> 1) & 7);
     int n;
     if (SWIGLU) n = row < BN / 2 ? min(n0 + row, N - 1) : up_offset + min(n0 + row - BN / 2, N - 1);
     else n = min(n0 + row, N - 1);
-    src[MW] = W + (size_t)n * K + seg * 8;
+    src[MW + d] = W + (size_t)n * K + seg * 8;
   }
   typedef __attribute__((address_space(3))) u32x4_t* lds_ptr_t;
   typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -606,8 +609,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
     for (int d = 0; d < MW; ++d)
       __builtin_amdgcn_global_load_lds((gptr_t)(src[d] + k0), (__attribute__((address_space(3))) void*)
                                        (buf + (wave * MW + d) * 64), 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((gptr_t)(src[MW] + k0), (__attribute__((address_space(3))) void*)
-                                     (buf + A_BYTES / 16 + wave * 64), 16, 0, 0);
+#pragma unroll
+    for (int d = 0; d < NWI; ++d)
+      __builtin_amdgcn_global_load_lds((gptr_t)(src[MW + d] + k0), (__attribute__((address_space(3))) void*)
+                                       (buf + A_BYTES / 16 + (wave * NWI + d) * 64), 16, 0, 0);
   };
 
 #pragma unroll
@@ -686,16 +691,16 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   }
 }
 
-template <int MW, int NB, typename TC, int EPI>
+template <int MW, int NT, int NB, typename TC, int EPI>
 static int launch_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                        hipStream_t stream) {
   constexpr int BM = 64 * MW;
-  constexpr int COLS = EPI == EPI_SWIGLU ? 32 : 64;
-  constexpr size_t lds_bytes = (size_t)NB * (BM * 128 + 64 * 128);
+  constexpr int COLS = EPI == EPI_SWIGLU ? 8 * NT : 16 * NT;
+  constexpr size_t lds_bytes = (size_t)NB * (BM + 16 * NT) * 128;
   static_assert(lds_bytes <= 160 * 1024, "the LDS of a compute unit");
   dim3 grid((N + COLS - 1) / COLS, parts, (M + BM - 1) / BM);
   if (grid.z > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
-  auto kernel = gemm_wide_kernel<MW, NB, TC, EPI>;
+  auto kernel = gemm_wide_kernel<MW, NT, NB, TC, EPI>;
   static bool allowed[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SA_ERR_ARG;
@@ -733,10 +738,19 @@ static bool takes_wide(int M, int N, int K, int parts) {
 template <typename TC, int EPI>
 static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                      hipStream_t stream) {
-  // one or two groups of 64 rows; the ring as deep as LDS allows up to five stages
+  // one or two groups of 64 rows of A; 64 rows of W a workgroup, or 128 where 64 would give more workgroups
+  // than there are compute units (K 4096, 2 x 14336 rows of W, 64 rows of A: 45 us against 60; the
+  // head over 128,256 rows at 128 rows of A: 161 against 180 with K 2048, 239 against 294 with K 4096);
+  // the ring as deep as measured to pay
   if constexpr (EPI != EPI_QKV_ROPE) {
-    if (M <= 64) return launch_wide<1, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
-    return launch_wide<2, 5, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+    const long long rows_w = EPI == EPI_SWIGLU ? 2ll * N : N;
+    const bool many = (rows_w + 63) / 64 * parts > compute_units();
+    if (M <= 64) {
+      if (many) return launch_wide<1, 8, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+      return launch_wide<1, 4, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+    }
+    if (many) return launch_wide<2, 8, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+    return launch_wide<2, 4, 5, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
   }
   return SA_ERR_ARG;
 }

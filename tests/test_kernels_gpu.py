@@ -629,7 +629,9 @@ def test_swiglu_bf16(M, I, K):
 @pytest.mark.parametrize("kind,M,N,K,parts", [
     # gate/up with SwiGLU: 17 to 128 rows, K whole stages of 64; widths that are no multiple of a workgroup's 32
     ("swiglu", 17, 40, 128, 1), ("swiglu", 33, 1000, 192, 1), ("swiglu", 64, 8192, 2048, 1),
-    ("swiglu", 100, 77, 256, 1), ("swiglu", 128, 8200, 320, 1), ("swiglu", 65, 12300, 4096, 1),
+    ("swiglu", 100, 77, 256, 1), ("swiglu", 128, 8200, 320, 1),
+    # so many weight rows that a workgroup takes 128 of them
+    ("swiglu", 65, 12300, 4096, 1), ("swiglu", 40, 9000, 128, 1), ("plain", 128, 20000, 128, 1), ("plain", 50, 33001, 256, 1),
     # the head: many rows of W, 48 rows and more (9 and more with a long K)
     ("plain", 48, 8200, 128, 1), ("plain", 64, 32064, 192, 1), ("plain", 100, 9001, 192, 1), ("plain", 9, 8200, 4096, 1),
     ("plain", 128, 8195, 2048, 1),

@@ -2,7 +2,7 @@
 // prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
 // Three kernels: gemm_skinny_kernel for one or two rows, gemm_mid_kernel for up to 128 (per pass),
 // and gemm_wide_kernel, which brings both operands into LDS without passing registers and takes
-// the products of 17 to 128 rows where that is faster (see pick_wide).
+// the products of up to 128 rows where that is faster (see takes_wide).
 //
 // The work is bound by reading W.  In the first, a wave owns RT tiles of 16 rows of W and walks a
 // slice of K in steps of 32; the KS waves of a workgroup split K between them and add their partial sums
@@ -716,23 +716,35 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
   return 0;
 }
 
-// Which products gemm_wide_kernel takes, from timings beside gemm_mid_kernel at the sizes of the
-// Llama-3 family with cold weights, 16 to 256 rows (in microseconds, wide against mid):
-//   gate/up + SwiGLU, K 2048, 2 x 8192 rows of W: 13.8 / 17.0 at 32 rows, 15.4 / 19.3 at 64, 18.7 / 26.1 at 128;
-//     K 4096, 2 x 14336: level up to 64 rows, 66 / 73 at 80, 73 / 82 at 128;
-//   down_proj in fp32 parts, K 8192: 9.6 / 10.0 at 32, 10.9 / 13.1 at 64, 15.0 / 17.6 at 128 (eight parts
-//     against four); K 14336: 24 / 28 at 32, 27 / 34 at 64, 43 / 52 at 128;
-//   o_proj, K 2048: 6.7 / 6.1 at 64, 9.6 / 8.5 at 128 (mid stays); K 4096: 10.9 / 12.3 at 64, 14.9 / 17.4 at 128;
-//   the head over 128,256 rows of W, K 2048: 116 / 111 at 32, 128 / 132 at 64, 154 / 165 at 96, 168 / 190 at 128;
-//     K 4096: 188 / 298 at 16, 223 / 301 at 64, 286 / 330 at 128.
-// At 16 rows and fewer gemm_mid_kernel is level or ahead everywhere but for that last matrix.
+// Which products gemm_wide_kernel takes, from timings beside the two kernels above at the sizes of the
+// Llama-3 family (widths 2048, 3072, 4096) with cold weights, 1 to 128 rows; in microseconds, this kernel
+// against the other:
+//   gate/up + SwiGLU: K 2048, 2 x 8192 rows of W: level up to 12 rows, 13.7 / 14.1 at 16, 13.7 / 16.7 at 32,
+//     14.5 / 18.6 at 64, 19.0 / 24.5 at 128; K 3072, 2 x 8192: 20.2 / 21.0 at one row, 20.1 / 23.4 at 16,
+//     22.5 / 27.8 at 64, 29.8 / 35.5 at 128; K 4096, 2 x 14336 (128 rows of W a workgroup): 45.3 / 48.6 at one
+//     row, 45.4 / 47.7 at 16, 45.8 / 54.8 at 64, 53.2 / 81.7 at 128;
+//   the head over 128,256 rows of W: K 2048: 99 / 95 at 8 rows, 118 / 118 at 48, 145 / 163 at 96, 159 / 185 at
+//     128; K 3072: 135 / 148 at one row, 139 / 153 at 16, 169 / 197 at 64, 210 / 266 at 128; K 4096: 177 / 204
+//     at one row, 176 / 290 at 12, 197 / 302 at 64, 238 / 319 at 128;
+//   narrow matrices in fp32 parts: down_proj K 8192, 2048 rows of W (eight parts against four): 8.9 / 8.4 at 8
+//     rows, 9.5 / 9.5 at 32, 10.8 / 12.3 at 64, 15.3 / 17.8 at 128; K 8192, 3072 rows (four parts): 12.6 /
+//     10.7 at one row, 12.3 / 12.9 at 4, 13.4 / 16.0 at 32, 15.9 / 21.2 at 64, 22.2 / 32.3 at 128; K 14336, 4096
+//     rows: level up to 8 rows, 23.0 / 27.6 at 32, 26.4 / 35.6 at 64, 48 / 53 at 128; o_proj K 2048: 5.4 / 4.2
+//     at 8 rows, 7.4 / 6.1 at 64, 10.5 / 8.7 at 128 (the other kernel stays); K 3072: 7.4 / 7.0 at one row,
+//     6.8 / 8.1 at 4, 9.4 / 14.1 at 64, 13.9 / 20.2 at 128; K 4096: 9.0 / 8.1 at one row, 9.0 / 9.2 at 8, 10.9 /
+//     14.7 at 64, 15.1 / 22.5 at 128.
+// So: the longer a workgroup's walk along K, the fewer rows it takes for this kernel to be ahead.
 template <typename TC, int EPI>
 static bool takes_wide(int M, int N, int K, int parts) {
-  if (EPI == EPI_QKV_ROPE || M > 128 || (K & 63) || parts < 1 || (K >> 6) % parts || (K >> 6) / parts < 2) return false;
-  if (EPI == EPI_SWIGLU) return M > 16;
-  if (N >= 8192) return parts == 1 && (M >= 48 || (K >= 4096 && M > 8));       // the head
-  // narrow matrices with a long K, cut into enough parts to give half the compute units a workgroup
-  return M > 16 && K >= 4096 && ((N + 63) / 64) * parts >= 128;
+  if (EPI == EPI_QKV_ROPE || M < 1 || M > 128 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
+  const int stages = (K >> 6) / parts;             // of a workgroup
+  if (stages < 2) return false;
+  if (EPI == EPI_SWIGLU) return K >= 3072 || M >= 16;
+  if (N >= 8192) return parts == 1 && (K >= 3072 || M >= 48);                    // the head
+  // narrow matrices: a walk of twelve stages and more, and enough parts to give half the compute units a
+  // workgroup; from three rows on for matrices of 24 M elements and more, above 32 rows for smaller ones
+  if (stages < 12 || ((N + 63) / 64) * parts < 128) return false;
+  return M > 32 || (M > 2 && (long long)N * K >= (24ll << 20));
 }
 
 template <typename TC, int EPI>
@@ -891,14 +903,14 @@ extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K & 7) || parts < 1) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
+  if (takes_wide<float, EPI_PLAIN>(M, N, K, parts)) {
+    if (c_dtype == SA_BF16 && parts == 1) return pick_wide<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, stream);
+    if (c_dtype == SA_F32) return pick_wide<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, stream);
+    return SA_ERR_UNSUPPORTED;
+  }
   if (!takes_skinny<float, EPI_PLAIN>(M, N, none)) {
-    const bool wide = takes_wide<float, EPI_PLAIN>(M, N, K, parts);
-    if (c_dtype == SA_BF16 && parts == 1)
-      return wide ? pick_wide<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, stream)
-                  : pick_mid<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
-    if (c_dtype == SA_F32)
-      return wide ? pick_wide<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, stream)
-                  : pick_mid<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
+    if (c_dtype == SA_BF16 && parts == 1) return pick_mid<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
+    if (c_dtype == SA_F32) return pick_mid<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
     return SA_ERR_UNSUPPORTED;
   }
   if (c_dtype == SA_BF16 && parts == 1) return pick_skinny<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);

@@ -472,22 +472,22 @@ def gemm_takes_wide(M: int, N: int, K: int, parts: int = 1, swiglu: bool = False
 
 def split_k_parts(M: int, N: int, K: int) -> int:
     """Into how many slices the inner dimension of a few-row product is cut across workgroups so
-    that a matrix with few rows still fills the chip: 1 means no cut.  One or two rows: a workgroup
-    takes 16 weight rows (about four workgroups per compute unit wanted, slices of at least 256); from three rows on
-    it takes 32 (one workgroup per compute unit wanted, slices of at least 512)."""
+    that a matrix with few rows still fills the chip: 1 means no cut.  Where the kernel with both
+    operands in LDS takes the product (64 weight rows a workgroup): as many as one round of workgroups
+    over the chip allows, slices of at least twelve stages of 64 columns.  Else, for one or two rows, a
+    workgroup takes 16 weight rows (about four workgroups per compute unit wanted, slices of at least
+    256); from three rows on it takes 32 (one workgroup per compute unit wanted, slices of at least 512)."""
     if N >= 8192:
         return 1
     cus = compute_units()
-    parts = 1
-    if 16 < M <= SKINNY_MAX_ROWS and K >= 4096 and K % 64 == 0:
-        # the kernel with both operands in LDS takes these (csrc/gemm_mfma.hip, takes_wide): 64 weight
-        # rows a workgroup, whole stages of 64 columns for every part
+    if M <= SKINNY_MAX_ROWS and K % 64 == 0:
         groups = -(-N // 64)
-        while parts < 8 and groups * parts < cus and K // (parts * 2) >= 512:
-            parts *= 2
-        if (K // 64) % parts == 0 and groups * parts >= 128:
-            return parts
         parts = 1
+        while parts < 8 and groups * parts * 2 <= cus and K // (64 * parts * 2) >= 12 and (K // 64) % (parts * 2) == 0:
+            parts *= 2
+        if gemm_takes_wide(M, N, K, parts):
+            return parts
+    parts = 1
     if M > 2:
         groups = -(-N // 32)
         while parts < 8 and groups * parts < cus and K // (parts * 2) >= 512:

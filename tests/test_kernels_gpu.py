@@ -636,11 +636,15 @@ def test_swiglu_bf16(M, I, K):
     ("plain", 48, 8200, 128, 1), ("plain", 64, 32064, 192, 1), ("plain", 100, 9001, 192, 1), ("plain", 9, 8200, 4096, 1),
     ("plain", 128, 8195, 2048, 1),
     # narrow matrices with a long K, in parts
-    ("parts", 32, 2048, 8192, 8), ("parts", 64, 4096, 4096, 4), ("parts", 70, 1664, 4480, 5), ("parts", 128, 2050, 8192, 8),
-    ("parts", 17, 4100, 14336, 2)])
+    ("parts", 40, 2048, 8192, 8), ("parts", 64, 4096, 4096, 4), ("parts", 70, 1664, 4480, 5), ("parts", 128, 2050, 8192, 8),
+    ("parts", 17, 4100, 14336, 2),
+    # a long inner dimension: from one row on (gate/up, the head), from three (narrow matrices)
+    ("swiglu", 1, 520, 3072, 1), ("swiglu", 5, 9000, 3136, 1), ("plain", 1, 8200, 3072, 1), ("plain", 3, 20000, 4096, 1),
+    ("parts", 3, 3072, 8192, 4)])
 def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
     """The sizes that `gemm_wide_kernel` takes (asserted), against the float64 product: row counts that are no
-    multiple of 16, widths that are no multiple of a workgroup's columns, one or two groups of 64 rows, parts."""
+    multiple of 16, widths that are no multiple of a workgroup's columns, one or two groups of 64 rows, 64 or
+    128 weight rows a workgroup, parts."""
     from serve_amd import ops
     assert ops.gemm_takes_wide(M, N, K, parts, swiglu=kind == "swiglu")
     a = rnd((M, K), torch.bfloat16, 14)
@@ -667,8 +671,7 @@ def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
         if N >= 2048:
             # the number of parts that the linear part chooses for such a matrix is one this kernel takes
             assert ops.gemm_takes_wide(M, N, K, ops.split_k_parts(M, N, K))
-    # rows beyond these sizes and inner sizes that are no whole stages stay with the other kernels
-    assert not ops.gemm_takes_wide(16, N, K, parts, swiglu=kind == "swiglu") or kind == "plain"
+    # more rows, and inner sizes that are no whole stages, stay with the other kernels
     assert not ops.gemm_takes_wide(129, N, K, parts) and not ops.gemm_takes_wide(M, N, K + 8, parts)
 
 

@@ -533,17 +533,21 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
 
 template <int MW, int NT, int NB, typename TC, int EPI>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
-                                                       TC* __restrict__ C, int M, int N, int K, int up_offset) {
+                                                       TC* __restrict__ C, int M, int N, int K, int up_offset,
+                                                       QkvRopeArgs qa) {
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
-  static_assert(EPI == EPI_PLAIN || EPI == EPI_SWIGLU, "the rotating epilogue stays with gemm_mid_kernel");
-  static_assert(NT == 4 || NT == 8, "tiles of 16 weight rows, 8 rows a wave and instruction; SwiGLU: half of the gate, half of up");
+  constexpr bool QKV = EPI == EPI_QKV_ROPE;
+  static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8, "tiles of 16 weight rows, 8 rows a wave and instruction");
+  static_assert(!SWIGLU || NT >= 2, "SwiGLU: half of the tiles are the gate's, half are up's");
   constexpr int BM = 64 * MW;
   constexpr int BN = 16 * NT;
   constexpr int A_BYTES = BM * 128;
   constexpr int STAGE_BYTES = A_BYTES + BN * 128;
   constexpr int COLS = SWIGLU ? BN / 2 : BN;       // output columns of a workgroup
-  constexpr int NWI = NT / 4;                      // weight loads per wave and stage
-  constexpr int ND = MW + NWI;                     // loads per wave and stage
+  // weight loads per stage: 2 NT instructions of 8 rows; with four tiles and more every wave issues NT / 4
+  // of them, with fewer the first 2 NT waves issue one each
+  constexpr int NWI = NT >= 4 ? NT / 4 : 1;
+  constexpr int ND = MW + NWI;
   static_assert(ND * (NB - 1) < 64, "the counter of loads in flight has six bits");
   static_assert(NB * STAGE_BYTES >= 4 * MW * NT * 4 * 64 * 4, "the sums of the second K half reuse the ring");
   extern __shared__ __attribute__((aligned(16))) u32x4_t wide_lds[];
@@ -556,6 +560,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   const int kh = wave >> 2;
   const int m0 = blockIdx.z * BM;
   const int n0 = blockIdx.x * COLS;
+  const bool has_w = NT >= 4 || wave < 2 * NT;     // (wave-uniform) whether this wave fetches weight rows
+  // the rotating epilogue: a tile holds eight dims of a head and their partners half a head further on
+  const int tph = QKV ? (qa.D >> 4) : 1;
+  const int tile0 = blockIdx.x * NT;
 
   const int nstages = (K >> 6) / gridDim.y;
   const int k_begin = blockIdx.y * nstages * 64;
@@ -580,11 +588,18 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   }
 #pragma unroll
   for (int d = 0; d < NWI; ++d) {
-    const int row = (wave * NWI + d) * 8 + (lane >> 3);
+    const int row = ((has_w ? wave : 0) * NWI + d) * 8 + (lane >> 3);       // of the workgroup's BN weight rows
     const int seg = (lane & 7) ^ ((row >> 1) & 7);
     int n;
-    if (SWIGLU) n = row < BN / 2 ? min(n0 + row, N - 1) : up_offset + min(n0 + row - BN / 2, N - 1);
-    else n = min(n0 + row, N - 1);
+    if (SWIGLU) {
+      n = row < BN / 2 ? min(n0 + row, N - 1) : up_offset + min(n0 + row - BN / 2, N - 1);
+    } else if (QKV) {
+      const int tile = tile0 + (row >> 4), cc = row & 15;
+      const int head = tile / tph, t16 = tile - head * tph;
+      n = head < qa.Hq + 2 * qa.Hk ? head * qa.D + t16 * 8 + (cc < 8 ? cc : (qa.D >> 1) + cc - 8) : 0;
+    } else {
+      n = min(n0 + row, N - 1);
+    }
     src[MW + d] = W + (size_t)n * K + seg * 8;
   }
   typedef __attribute__((address_space(3))) u32x4_t* lds_ptr_t;
@@ -595,6 +610,16 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   const uint32_t slot16 = (uint32_t)(((kh * 4 + g) ^ ((c >> 1) & 7)) * 16);
   const uint32_t a_addr = lds_base + (uint32_t)((mw * MW * 16 + c) * 128) + slot16;
   const uint32_t w_addr = lds_base + A_BYTES + (uint32_t)(c * 128) + slot16;
+
+  // what the rotating epilogue needs besides the sums, fetched beside the first stages
+  QkvLane<MW> ql[QKV ? NT : 1] = {};
+  if (QKV && kh == 0) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int tile = tile0 + nt, head = tile / tph;
+      ql[nt] = load_qkv_lane<MW>(qa, M, m0 + mw * MW * 16, head, tile - head * tph, g, c);
+    }
+  }
 
   floatx4_t acc[MW][NT];
 #pragma unroll
@@ -609,16 +634,20 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
     for (int d = 0; d < MW; ++d)
       __builtin_amdgcn_global_load_lds((gptr_t)(src[d] + k0), (__attribute__((address_space(3))) void*)
                                        (buf + (wave * MW + d) * 64), 16, 0, 0);
+    if (has_w) {
 #pragma unroll
-    for (int d = 0; d < NWI; ++d)
-      __builtin_amdgcn_global_load_lds((gptr_t)(src[MW + d] + k0), (__attribute__((address_space(3))) void*)
-                                       (buf + A_BYTES / 16 + (wave * NWI + d) * 64), 16, 0, 0);
+      for (int d = 0; d < NWI; ++d)
+        __builtin_amdgcn_global_load_lds((gptr_t)(src[MW + d] + k0), (__attribute__((address_space(3))) void*)
+                                         (buf + A_BYTES / 16 + (wave * NWI + d) * 64), 16, 0, 0);
+    }
   };
 
 #pragma unroll
   for (int i = 0; i < NB - 1; ++i) fetch(i);
   for (int s = 0; s < nstages; ++s) {
-    SA_WAIT_VMCNT(ND * (NB - 2));              // this wave's part of stage s lies in LDS
+    // this wave's part of stage s lies in LDS: all of its loads but those of the NB - 2 stages after it have landed
+    if (has_w) SA_WAIT_VMCNT(ND * (NB - 2));
+    else SA_WAIT_VMCNT(MW * (NB - 2));
     __builtin_amdgcn_s_barrier();              // everybody's does, and everybody has read stage s - 1
     fetch(s + NB - 1);
     const uint32_t boff = (uint32_t)((s % NB) * STAGE_BYTES);
@@ -662,6 +691,19 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
     for (int nt = 0; nt < NT; ++nt)
       acc[mt][nt] += *reinterpret_cast<const floatx4_t*>(&red[((((mw * MW + mt) * NT + nt) * 64) + lane) * 4]);
 
+  if constexpr (QKV) {
+    // tile by tile through the epilogue of the kernels above: rotation, q to its buffer, k and v into the cache
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int tile = tile0 + nt, head = tile / tph, t16 = tile - head * tph;
+      if (head >= qa.Hq + 2 * qa.Hk) continue;             // (wave-uniform)
+      floatx4_t one[1][MW];
+#pragma unroll
+      for (int mt = 0; mt < MW; ++mt) one[0][mt] = acc[mt][nt];
+      store_tiles<1, MW, TC, EPI>(one, C, M, N, m0 + mw * MW * 16, head * qa.D + t16 * 8, head, t16, qa, ql[nt], g, c);
+    }
+    return;
+  }
   // lane l holds C[m = row tile's row l % 16][n = 4 (l / 16) .. + 3] of every tile pair
 #pragma unroll
   for (int mt = 0; mt < MW; ++mt) {
@@ -693,25 +735,29 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
 
 template <int MW, int NT, int NB, typename TC, int EPI>
 static int launch_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
-                       hipStream_t stream) {
+                       const QkvRopeArgs& qa, hipStream_t stream) {
   constexpr int BM = 64 * MW;
   constexpr int COLS = EPI == EPI_SWIGLU ? 8 * NT : 16 * NT;
   constexpr size_t lds_bytes = (size_t)NB * (BM + 16 * NT) * 128;
   static_assert(lds_bytes <= 160 * 1024, "the LDS of a compute unit");
-  dim3 grid((N + COLS - 1) / COLS, parts, (M + BM - 1) / BM);
+  unsigned gx = (N + COLS - 1) / COLS;
+  if (EPI == EPI_QKV_ROPE) gx = ((qa.Hq + 2 * qa.Hk) * (qa.D >> 4) + NT - 1) / NT;
+  dim3 grid(gx, parts, (M + BM - 1) / BM);
   if (grid.z > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
   auto kernel = gemm_wide_kernel<MW, NT, NB, TC, EPI>;
-  static bool allowed[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SA_ERR_ARG;
-  if (!allowed[dev]) {        // more dynamic LDS than a kernel gets without asking
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return (int)e;
-    allowed[dev] = true;
+  if (lds_bytes > 64 * 1024) {  // more dynamic LDS than a kernel gets without asking
+    static bool allowed[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SA_ERR_ARG;
+    if (!allowed[dev]) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+      if (e != hipSuccess) return (int)e;
+      allowed[dev] = true;
+    }
   }
   hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, stream, (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K,
-                     up_offset);
+                     up_offset, qa);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -733,12 +779,17 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
 //     at 8 rows, 7.4 / 6.1 at 64, 10.5 / 8.7 at 128 (the other kernel stays); K 3072: 7.4 / 7.0 at one row,
 //     6.8 / 8.1 at 4, 9.4 / 14.1 at 64, 13.9 / 20.2 at 128; K 4096: 9.0 / 8.1 at one row, 9.0 / 9.2 at 8, 10.9 /
 //     14.7 at 64, 15.1 / 22.5 at 128.
+//   q/k/v + rotation + cache write (16 weight rows a workgroup, 32 where 16 would give more workgroups than
+//     compute units): K 2048, 3072 rows of W: 10.0 / 6.0 at one row, 10.2 / 8.4 at 32, 10.7 / 11.5 at 64, 13.6 / 17.3
+//     at 128; K 3072, 5120 rows: 15.8 / 16.5 at 48, 16.0 / 19.4 at 64, 21.8 / 28.5 at 128; K 4096, 6144 rows: 19.6 /
+//     19.5 at 48, 20.5 / 22.2 at 64, 26.8 / 33.5 at 128.
 // So: the longer a workgroup's walk along K, the fewer rows it takes for this kernel to be ahead.
 template <typename TC, int EPI>
 static bool takes_wide(int M, int N, int K, int parts) {
-  if (EPI == EPI_QKV_ROPE || M < 1 || M > 128 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
+  if (M < 1 || M > 128 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
   const int stages = (K >> 6) / parts;             // of a workgroup
   if (stages < 2) return false;
+  if (EPI == EPI_QKV_ROPE) return M >= 64;
   if (EPI == EPI_SWIGLU) return K >= 3072 || M >= 16;
   if (N >= 8192) return parts == 1 && (K >= 3072 || M >= 48);                    // the head
   // narrow matrices: a walk of twelve stages and more, and enough parts to give half the compute units a
@@ -749,21 +800,33 @@ static bool takes_wide(int M, int N, int K, int parts) {
 
 template <typename TC, int EPI>
 static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
-                     hipStream_t stream) {
+                     const QkvRopeArgs& qa, hipStream_t stream) {
   // one or two groups of 64 rows of A; 64 rows of W a workgroup, or 128 where 64 would give more workgroups
   // than there are compute units (K 4096, 2 x 14336 rows of W, 64 rows of A: 45 us against 60; the
   // head over 128,256 rows at 128 rows of A: 161 against 180 with K 2048, 239 against 294 with K 4096);
   // the ring as deep as measured to pay
-  if constexpr (EPI != EPI_QKV_ROPE) {
+#define GO(MW, NT, NB) return launch_wide<MW, NT, NB, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
+  if constexpr (EPI == EPI_QKV_ROPE) {
+    // few weight rows in all: 16 of them a workgroup, or 32 where that still gives every compute unit one
+    const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
+    const bool two = tiles > compute_units();
+    if (M <= 64) {
+      if (two) GO(1, 2, 6);
+      GO(1, 1, 6);
+    }
+    if (two) GO(2, 2, 5);
+    GO(2, 1, 5);
+  } else {
     const long long rows_w = EPI == EPI_SWIGLU ? 2ll * N : N;
     const bool many = (rows_w + 63) / 64 * parts > compute_units();
     if (M <= 64) {
-      if (many) return launch_wide<1, 8, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
-      return launch_wide<1, 4, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+      if (many) GO(1, 8, 4);
+      GO(1, 4, 4);
     }
-    if (many) return launch_wide<2, 8, 4, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
-    return launch_wide<2, 4, 5, TC, EPI>(A, W, C, M, N, K, up_offset, parts, stream);
+    if (many) GO(2, 8, 4);
+    GO(2, 4, 5);
   }
+#undef GO
   return SA_ERR_ARG;
 }
 
@@ -888,10 +951,11 @@ static int pick_skinny(const void* A, const void* W, void* C, int M, int N, int 
   return SA_ERR_ARG;
 }
 
-// whether a product of these sizes goes to gemm_wide_kernel (epi: EPI_PLAIN or EPI_SWIGLU, for which N
-// is the number of gate rows): for the caller's choice of `parts`, and for tests
+// whether a product of these sizes goes to gemm_wide_kernel (epi: EPI_PLAIN, EPI_SWIGLU, for which N is the
+// number of gate rows, or EPI_QKV_ROPE): for the caller's choice of `parts`, and for tests
 extern "C" int sa_gemm_bf16_takes_wide(int epi, int M, int N, int K, int parts) {
   if (epi == EPI_SWIGLU) return takes_wide<bf16_t, EPI_SWIGLU>(M, N, K, parts) ? 1 : 0;
+  if (epi == EPI_QKV_ROPE) return takes_wide<bf16_t, EPI_QKV_ROPE>(M, N, K, parts) ? 1 : 0;
   if (epi == EPI_PLAIN) return takes_wide<float, EPI_PLAIN>(M, N, K, parts) ? 1 : 0;
   return 0;
 }
@@ -904,8 +968,8 @@ extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_
   if (K <= 0 || (K & 7) || parts < 1) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
   if (takes_wide<float, EPI_PLAIN>(M, N, K, parts)) {
-    if (c_dtype == SA_BF16 && parts == 1) return pick_wide<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, stream);
-    if (c_dtype == SA_F32) return pick_wide<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, stream);
+    if (c_dtype == SA_BF16 && parts == 1) return pick_wide<bf16_t, EPI_PLAIN>(A, W, C, M, N, K, 0, 1, none, stream);
+    if (c_dtype == SA_F32) return pick_wide<float, EPI_PLAIN>(A, W, C, M, N, K, 0, parts, none, stream);
     return SA_ERR_UNSUPPORTED;
   }
   if (!takes_skinny<float, EPI_PLAIN>(M, N, none)) {
@@ -924,7 +988,7 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
   if (M <= 0 || I <= 0) return 0;
   if (K <= 0 || (K & 7)) return SA_ERR_ARG;
   const QkvRopeArgs none = {};
-  if (takes_wide<bf16_t, EPI_SWIGLU>(M, I, K, 1)) return pick_wide<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, stream);
+  if (takes_wide<bf16_t, EPI_SWIGLU>(M, I, K, 1)) return pick_wide<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   if (!takes_skinny<bf16_t, EPI_SWIGLU>(M, I, none)) return pick_mid<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   return pick_skinny<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
 }
@@ -938,6 +1002,7 @@ extern "C" int sa_gemm_bf16_qkv_rope(const void* A, const void* W, void* Q, cons
   if (M <= 0) return 0;
   if (K <= 0 || (K & 7) || Hq <= 0 || Hk <= 0 || D <= 0 || (D & 15) || page_size <= 0) return SA_ERR_ARG;
   const QkvRopeArgs qa = {positions, inv_freq, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size};
+  if (takes_wide<bf16_t, EPI_QKV_ROPE>(M, 0, K, 1)) return pick_wide<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   if (!takes_skinny<bf16_t, EPI_QKV_ROPE>(M, 0, qa)) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   return pick_skinny<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
 }

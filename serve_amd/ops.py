@@ -8,6 +8,7 @@ library that cannot be compiled is an error (`serve_amd.csrc.build.BuildError`).
 from __future__ import annotations
 
 import ctypes
+import functools
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
@@ -470,6 +471,7 @@ def gemm_takes_wide(M: int, N: int, K: int, parts: int = 1, swiglu: bool = False
     return bool(lib.sa_gemm_bf16_takes_wide(c_int(1 if swiglu else 0), c_int(M), c_int(N), c_int(K), c_int(parts)))
 
 
+@functools.lru_cache(maxsize=4096)
 def split_k_parts(M: int, N: int, K: int) -> int:
     """Into how many slices the inner dimension of a few-row product is cut across workgroups so
     that a matrix with few rows still fills the chip: 1 means no cut.  Where the kernel with both

@@ -732,7 +732,12 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
                                              (64, 28, 2, 128, 16, 264), (3, 60, 4, 64, 16, 64),
                                              # 65 to 128 rows
                                              (65, 32, 8, 64, 16, 2048), (128, 3, 1, 96, 16, 72), (100, 24, 8, 128, 16, 264),
-                                             (77, 4, 2, 16, 8, 40), (90, 24, 8, 128, 16, 136), (110, 28, 2, 128, 16, 72)])
+                                             (77, 4, 2, 16, 8, 40), (90, 24, 8, 128, 16, 136), (110, 28, 2, 128, 16, 72),
+                                             # 64 rows and more with an inner size of whole stages of 64: both operands
+                                             # through LDS, 16 weight rows a workgroup, or 32 with more than 256 tiles
+                                             # (an odd number of them: the last workgroup has one)
+                                             (64, 32, 8, 64, 16, 2048), (100, 32, 8, 128, 16, 256), (64, 5, 1, 48, 16, 128),
+                                             (128, 40, 8, 128, 16, 192), (70, 3, 1, 80, 16, 128), (64, 85, 1, 48, 16, 128)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
     P = 7 if M <= 64 else 20

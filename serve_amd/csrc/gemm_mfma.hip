@@ -2,7 +2,7 @@
 // prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
 // Three kernels: gemm_skinny_kernel for one or two rows, gemm_mid_kernel for up to 128 (per pass),
 // and gemm_wide_kernel, which brings both operands into LDS without passing registers and takes
-// the products of up to 128 rows where that is faster (see takes_wide).
+// the products of up to 192 rows where that is faster (see takes_wide).
 //
 // The work is bound by reading W.  In the first, a wave owns RT tiles of 16 rows of W and walks a
 // slice of K in steps of 32; the KS waves of a workgroup split K between them and add their partial sums
@@ -783,15 +783,20 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
 //     compute units): K 2048, 3072 rows of W: 10.0 / 6.0 at one row, 10.2 / 8.4 at 32, 10.7 / 11.5 at 64, 13.6 / 17.3
 //     at 128; K 3072, 5120 rows: 15.8 / 16.5 at 48, 16.0 / 19.4 at 64, 21.8 / 28.5 at 128; K 4096, 6144 rows: 19.6 /
 //     19.5 at 48, 20.5 / 22.2 at 64, 26.8 / 33.5 at 128.
+// 129 to 192 rows, against the BLAS library (and its SwiGLU pass): gate/up 22.7 / 30.6 at 160 rows and 24.4 / 31.0
+// at 192 with K 2048, 34.5 / 36.4 and 37.2 / 40.6 with K 3072, 62.2 / 65.8 and 64.0 / 68.7 with K 4096; down_proj
+// 18.4 / 25.7 and 20.8 / 26.9 (K 8192, 2048 rows), 26.0 / 27.6 and 29.2 / 58.5 (3072 rows), 57.4 / 83.4 and 64.9 /
+// 102.6 (K 14336); o_proj 15.9 / 16.6 and 17.8 / 26.6 (K 3072), 17.9 / 26.7 and 19.5 / 32.2 (K 4096).  Beyond 192
+// rows the library is ahead for most of them, and for the head from 129 on.
 // So: the longer a workgroup's walk along K, the fewer rows it takes for this kernel to be ahead.
 template <typename TC, int EPI>
 static bool takes_wide(int M, int N, int K, int parts) {
-  if (M < 1 || M > 128 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
+  if (M < 1 || M > 192 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
   const int stages = (K >> 6) / parts;             // of a workgroup
   if (stages < 2) return false;
-  if (EPI == EPI_QKV_ROPE) return M >= 64;
+  if (EPI == EPI_QKV_ROPE) return M >= 64 && M <= 128;
   if (EPI == EPI_SWIGLU) return K >= 3072 || M >= 16;
-  if (N >= 8192) return parts == 1 && (K >= 3072 || M >= 48);                    // the head
+  if (N >= 8192) return parts == 1 && M <= 128 && (K >= 3072 || M >= 48);        // the head
   // narrow matrices: a walk of twelve stages and more, and enough parts to give half the compute units a
   // workgroup; from three rows on for matrices of 24 M elements and more, above 32 rows for smaller ones
   if (stages < 12 || ((N + 63) / 64) * parts < 128) return false;
@@ -801,7 +806,7 @@ static bool takes_wide(int M, int N, int K, int parts) {
 template <typename TC, int EPI>
 static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                      const QkvRopeArgs& qa, hipStream_t stream) {
-  // one or two groups of 64 rows of A; 64 rows of W a workgroup, or 128 where 64 would give more workgroups
+  // one to three groups of 64 rows of A; 64 rows of W a workgroup, or 128 where 64 would give more workgroups
   // than there are compute units (K 4096, 2 x 14336 rows of W, 64 rows of A: 45 us against 60; the
   // head over 128,256 rows at 128 rows of A: 161 against 180 with K 2048, 239 against 294 with K 4096);
   // the ring as deep as measured to pay
@@ -823,8 +828,12 @@ static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K,
       if (many) GO(1, 8, 4);
       GO(1, 4, 4);
     }
-    if (many) GO(2, 8, 4);
-    GO(2, 4, 5);
+    if (M <= 128) {
+      if (many) GO(2, 8, 4);
+      GO(2, 4, 5);
+    }
+    if (many) GO(3, 8, 3);
+    GO(3, 4, 4);
   }
 #undef GO
   return SA_ERR_ARG;

@@ -23,7 +23,7 @@ from ..parts.base import Runtime
 from .batch import INERT, Segment, StepLayout, context_from, plan_step
 
 # padded batch sizes for which decode-only steps are captured into graphs
-GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
+GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256)
 # more rows than that are replayed from graphs only where nobody asks for the logits (steps launched
 # ahead of the host, which sample on the device): such a graph keeps no [rows, vocabulary] buffer
 ASYNC_GRAPH_BATCHES = GRAPH_BATCHES + (384, 512)

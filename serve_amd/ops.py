@@ -429,6 +429,7 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Opti
 # library's: the few-row kernel would read its 128 rows of activations once per 64 weight rows
 WIDE_OUTPUT = 65536
 SKINNY_MAX_ROWS = 128         # above this the weights would be streamed more than once per product
+WIDE_MAX_ROWS = 192           # ... but for the kernel with both operands in LDS, where it is ahead of the library
 
 
 def _aligned16(*tensors: torch.Tensor) -> bool:
@@ -464,6 +465,7 @@ def gemm_bf16_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tor
     return out
 
 
+@functools.lru_cache(maxsize=4096)
 def gemm_takes_wide(M: int, N: int, K: int, parts: int = 1, swiglu: bool = False) -> bool:
     """Whether the few-row product of these sizes runs as the kernel that keeps both operands in LDS
     (for SwiGLU, N is the number of gate rows)."""
@@ -482,7 +484,7 @@ def split_k_parts(M: int, N: int, K: int) -> int:
     if N >= 8192:
         return 1
     cus = compute_units()
-    if M <= SKINNY_MAX_ROWS and K % 64 == 0:
+    if M <= WIDE_MAX_ROWS and K % 64 == 0:
         groups = -(-N // 64)
         parts = 1
         while parts < 8 and groups * parts * 2 <= cus and K // (64 * parts * 2) >= 12 and (K // 64) % (parts * 2) == 0:
@@ -538,7 +540,10 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
     """bf16 product: the weight-streaming kernels for few rows, the BLAS library for many (the
     reference leaves all of its products to the library, serve/model.py:80-82,95,97,159); both
     write bf16 or fp32."""
-    if a.shape[0] <= SKINNY_MAX_ROWS and not (a.shape[0] > 64 and w.shape[0] >= WIDE_OUTPUT):
+    M = a.shape[0]
+    if M <= SKINNY_MAX_ROWS and not (M > 64 and w.shape[0] >= WIDE_OUTPUT):
+        return gemm_bf16_skinny(a, w, out)
+    if M <= WIDE_MAX_ROWS and gemm_takes_wide(M, w.shape[0], a.shape[1], 1):
         return gemm_bf16_skinny(a, w, out)
     return gemm_bf16_library(a, w, out)
 

@@ -26,13 +26,15 @@ def linear(a: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     M = a.shape[0]
     N = w.shape[0]
     if (partial_ok and out is None and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-            and 0 < M <= ops.SKINNY_MAX_ROWS):
+            and 0 < M <= ops.WIDE_MAX_ROWS):
         # few rows: the product stays fp32 on its way into the residual stream, in one or more parts
+        # (above SKINNY_MAX_ROWS only where the kernel with both operands in LDS takes it)
         parts = ops.split_k_parts(M, N, a.shape[1])
-        out = torch.empty((parts, M, N), dtype=torch.float32, device=a.device)
-        if ops.mfma_gemm_available(a, w, out):
-            return ops.gemm_bf16_skinny(a, w, out)
-        out = None
+        if M <= ops.SKINNY_MAX_ROWS or ops.gemm_takes_wide(M, N, a.shape[1], parts):
+            out = torch.empty((parts, M, N), dtype=torch.float32, device=a.device)
+            if ops.mfma_gemm_available(a, w, out):
+                return ops.gemm_bf16_skinny(a, w, out)
+            out = None
     if partial_ok and out is None and out_dtype in (None, torch.float32) and ops.gemm_f32_mid_available(a, w):
         # float32, a few dozen rows: a narrow matrix fills the chip only with its inner dimension cut
         parts = ops.f32_mid_parts(M, N, a.shape[1])

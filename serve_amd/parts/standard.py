@@ -239,8 +239,10 @@ class SwiGLU(Part):
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         a = self.rt.empty((h.shape[0], self.intermediate_size))
-        if (h.shape[0] <= ops.SKINNY_MAX_ROWS and h.dtype == torch.bfloat16
-                and self.w_gate_up.dtype == torch.bfloat16 and self.hidden_size % 8 == 0):
+        M = h.shape[0]
+        if (h.dtype == torch.bfloat16 and self.w_gate_up.dtype == torch.bfloat16 and self.hidden_size % 8 == 0
+                and (M <= ops.SKINNY_MAX_ROWS or (M <= ops.WIDE_MAX_ROWS and ops.gemm_takes_wide(
+                    M, self.intermediate_size, self.hidden_size, 1, swiglu=True)))):
             ops.swiglu_bf16(h, self.w_gate_up, a)          # product and gate in one kernel
         else:
             gu = linear(h, self.w_gate_up)

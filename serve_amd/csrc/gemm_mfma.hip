@@ -2,7 +2,7 @@
 // prompt portions): C[M, N] = A[M, K] * W[N, K]^T, fp32 accumulation, weights streamed once.
 // Three kernels: gemm_skinny_kernel for one or two rows, gemm_mid_kernel for up to 128 (per pass),
 // and gemm_wide_kernel, which brings both operands into LDS without passing registers and takes
-// the products of up to 192 rows where that is faster (see takes_wide).
+// the products of up to 256 rows where that is faster (see takes_wide).
 //
 // The work is bound by reading W.  In the first, a wave owns RT tiles of 16 rows of W and walks a
 // slice of K in steps of 32; the KS waves of a workgroup split K between them and add their partial sums
@@ -787,15 +787,19 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
 // at 192 with K 2048, 34.5 / 36.4 and 37.2 / 40.6 with K 3072, 62.2 / 65.8 and 64.0 / 68.7 with K 4096; down_proj
 // 18.4 / 25.7 and 20.8 / 26.9 (K 8192, 2048 rows), 26.0 / 27.6 and 29.2 / 58.5 (3072 rows), 57.4 / 83.4 and 64.9 /
 // 102.6 (K 14336); o_proj 15.9 / 16.6 and 17.8 / 26.6 (K 3072), 17.9 / 26.7 and 19.5 / 32.2 (K 4096).  Beyond 192
-// rows the library is ahead for most of them, and for the head from 129 on.
+// rows the library is ahead for most of them (and for the head from 129 on), but not for gate/up of the smaller
+// models: 26.9 / 32.8 at 224 rows and 28.2 / 34.5 at 256 with K 2048, 40.4 / 44.6 and 42.3 / 46.7 with K 3072
+// (K 4096, 2 x 14336 rows: 78 / 75 and 81 / 78).
 // So: the longer a workgroup's walk along K, the fewer rows it takes for this kernel to be ahead.
 template <typename TC, int EPI>
 static bool takes_wide(int M, int N, int K, int parts) {
-  if (M < 1 || M > 192 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
+  if (M < 1 || M > 256 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
   const int stages = (K >> 6) / parts;             // of a workgroup
   if (stages < 2) return false;
   if (EPI == EPI_QKV_ROPE) return M >= 64 && M <= 128;
-  if (EPI == EPI_SWIGLU) return K >= 3072 || M >= 16;
+  // gate/up: beyond 192 rows only for matrices of up to 64 M elements, for which the library's fixed costs weigh most
+  if (EPI == EPI_SWIGLU) return (K >= 3072 || M >= 16) && (M <= 192 || 2ll * N * K <= (64ll << 20));
+  if (M > 192) return false;
   if (N >= 8192) return parts == 1 && M <= 128 && (K >= 3072 || M >= 48);        // the head
   // narrow matrices: a walk of twelve stages and more, and enough parts to give half the compute units a
   // workgroup; from three rows on for matrices of 24 M elements and more, above 32 rows for smaller ones
@@ -806,7 +810,7 @@ static bool takes_wide(int M, int N, int K, int parts) {
 template <typename TC, int EPI>
 static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                      const QkvRopeArgs& qa, hipStream_t stream) {
-  // one to three groups of 64 rows of A; 64 rows of W a workgroup, or 128 where 64 would give more workgroups
+  // one to four groups of 64 rows of A; 64 rows of W a workgroup, or 128 where 64 would give more workgroups
   // than there are compute units (K 4096, 2 x 14336 rows of W, 64 rows of A: 45 us against 60; the
   // head over 128,256 rows at 128 rows of A: 161 against 180 with K 2048, 239 against 294 with K 4096);
   // the ring as deep as measured to pay
@@ -832,8 +836,12 @@ static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K,
       if (many) GO(2, 8, 4);
       GO(2, 4, 5);
     }
-    if (many) GO(3, 8, 3);
-    GO(3, 4, 4);
+    if (M <= 192) {
+      if (many) GO(3, 8, 3);
+      GO(3, 4, 4);
+    }
+    if (many) GO(4, 8, 3);
+    GO(4, 4, 3);
   }
 #undef GO
   return SA_ERR_ARG;

@@ -429,7 +429,7 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], keys: Opti
 # library's: the few-row kernel would read its 128 rows of activations once per 64 weight rows
 WIDE_OUTPUT = 65536
 SKINNY_MAX_ROWS = 128         # above this the weights would be streamed more than once per product
-WIDE_MAX_ROWS = 192           # ... but for the kernel with both operands in LDS, where it is ahead of the library
+WIDE_MAX_ROWS = 256           # ... but for the kernel with both operands in LDS, where it is ahead of the library
 
 
 def _aligned16(*tensors: torch.Tensor) -> bool:

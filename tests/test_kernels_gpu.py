@@ -643,7 +643,9 @@ def test_swiglu_bf16(M, I, K):
     ("parts", 3, 3072, 8192, 4),
     # 129 to 192 rows: three groups of 64
     ("swiglu", 160, 1000, 192, 1), ("swiglu", 192, 9000, 128, 1), ("swiglu", 130, 8192, 2048, 1),
-    ("parts", 150, 2048, 8192, 8), ("parts", 192, 4096, 4096, 4)])
+    ("parts", 150, 2048, 8192, 8), ("parts", 192, 4096, 4096, 4),
+    # gate/up of a small model up to 256 rows: four groups
+    ("swiglu", 256, 8192, 2048, 1), ("swiglu", 200, 1000, 192, 1), ("swiglu", 250, 8200, 3072, 1)])
 def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
     """The sizes that `gemm_wide_kernel` takes (asserted), against the float64 product: row counts that are no
     multiple of 16, widths that are no multiple of a workgroup's columns, one or two groups of 64 rows, 64 or
@@ -675,7 +677,7 @@ def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
             # the number of parts that the linear part chooses for such a matrix is one this kernel takes
             assert ops.gemm_takes_wide(M, N, K, ops.split_k_parts(M, N, K))
     # more rows, and inner sizes that are no whole stages, stay with the other kernels
-    assert not ops.gemm_takes_wide(193, N, K, parts) and not ops.gemm_takes_wide(M, N, K + 8, parts)
+    assert not ops.gemm_takes_wide(257, N, K, parts) and not ops.gemm_takes_wide(M, N, K + 8, parts)
 
 
 def test_kernels_refuse_what_they_do_not_take():

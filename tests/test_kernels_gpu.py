@@ -635,6 +635,10 @@ def test_swiglu_bf16(M, I, K):
     # the head: many rows of W, 48 rows and more (9 and more with a long K)
     ("plain", 48, 8200, 128, 1), ("plain", 64, 32064, 192, 1), ("plain", 100, 9001, 192, 1), ("plain", 9, 8200, 4096, 1),
     ("plain", 128, 8195, 2048, 1),
+    # a vocabulary of 64 K rows and more: 256 weight rows a workgroup, from 8 rows on (one and two groups of 64
+    # rows; a width that is no multiple of 256, of 4, of anything; a long K, where only more rows take them)
+    ("plain", 8, 65792, 128, 1), ("plain", 40, 65543, 192, 1), ("plain", 100, 70000, 128, 1), ("plain", 128, 65600, 256, 1),
+    ("plain", 48, 65540, 3072, 1), ("plain", 72, 65536, 4096, 1),
     # narrow matrices with a long K, in parts
     ("parts", 40, 2048, 8192, 8), ("parts", 64, 4096, 4096, 4), ("parts", 70, 1664, 4480, 5), ("parts", 128, 2050, 8192, 8),
     ("parts", 17, 4100, 14336, 2),

@@ -535,7 +535,7 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
 // read from the last row and their sums never stored.
 #define SA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
 
-template <int MW, int NT, int NB, typename TC, int EPI>
+template <int MW, int NT, int NB, typename TC, int EPI, int SPB = 1>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                        TC* __restrict__ C, int M, int N, int K, int up_offset,
                                                        QkvRopeArgs qa) {
@@ -553,6 +553,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   constexpr int NWI = NT >= 4 ? NT / 4 : 1;
   constexpr int ND = MW + NWI;
   static_assert(ND * (NB - 1) < 64, "the counter of loads in flight has six bits");
+  static_assert(SPB >= 1 && NB % SPB == 0 && NB >= 2 * SPB, "SPB stages between two barriers, in a ring of whole groups of them");
   static_assert(NB * STAGE_BYTES >= 4 * MW * NT * 4 * 64 * 4, "the sums of the second K half reuse the ring");
   extern __shared__ __attribute__((aligned(16))) u32x4_t wide_lds[];
 
@@ -646,34 +647,46 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
     }
   };
 
+  // SPB stages between two barriers (two where a stage is so little work, one product a wave, that the
+  // barrier and the trip through LDS are what a stage takes; the launcher then gives an even number of stages)
 #pragma unroll
-  for (int i = 0; i < NB - 1; ++i) fetch(i);
-  for (int s = 0; s < nstages; ++s) {
-    // this wave's part of stage s lies in LDS: all of its loads but those of the NB - 2 stages after it have landed
-    if (has_w) SA_WAIT_VMCNT(ND * (NB - 2));
-    else SA_WAIT_VMCNT(MW * (NB - 2));
-    __builtin_amdgcn_s_barrier();              // everybody's does, and everybody has read stage s - 1
-    fetch(s + NB - 1);
-    const uint32_t boff = (uint32_t)((s % NB) * STAGE_BYTES);
+  for (int i = 0; i < NB - SPB; ++i) fetch(i);
+  for (int s = 0; s < nstages; s += SPB) {
+    // this wave's part of stages s .. s + SPB - 1 lies in LDS: all of its loads but those of the NB - 2 SPB
+    // stages after them have landed
+    if (has_w) SA_WAIT_VMCNT(ND * (NB - 2 * SPB));
+    else SA_WAIT_VMCNT(MW * (NB - 2 * SPB));
+    __builtin_amdgcn_s_barrier();              // everybody's does, and everybody has read the stages before s
+#pragma unroll
+    for (int u = 0; u < SPB; ++u) fetch(s + NB - SPB + u);
     // (the reads are written as instructions of their own: the compiler does not see the loads
     // into LDS as stores, and would otherwise wait for all of them before every read)
-    Frag af[MW], wf[NT];
+    Frag af[SPB][MW], wf[SPB][NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wf[nt].r) : "v"(w_addr + boff), "n"(nt * 16 * 128));
-#pragma unroll
-    for (int mt = 0; mt < MW; ++mt)
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[mt].r) : "v"(a_addr + boff), "n"(mt * 16 * 128));
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) asm volatile("" : "+v"(wf[nt].r));
-#pragma unroll
-    for (int mt = 0; mt < MW; ++mt) asm volatile("" : "+v"(af[mt].r));
-#pragma unroll
-    for (int mt = 0; mt < MW; ++mt)
+    for (int u = 0; u < SPB; ++u) {
+      const uint32_t boff = (uint32_t)(((s + u) % NB) * STAGE_BYTES);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt].v, af[mt].v, acc[mt][nt], 0, 0, 0);
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wf[u][nt].r) : "v"(w_addr + boff), "n"(nt * 16 * 128));
+#pragma unroll
+      for (int mt = 0; mt < MW; ++mt)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[u][mt].r) : "v"(a_addr + boff), "n"(mt * 16 * 128));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < SPB; ++u) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) asm volatile("" : "+v"(wf[u][nt].r));
+#pragma unroll
+      for (int mt = 0; mt < MW; ++mt) asm volatile("" : "+v"(af[u][mt].r));
+    }
+#pragma unroll
+    for (int u = 0; u < SPB; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MW; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][nt].v, af[u][mt].v, acc[mt][nt], 0, 0, 0);
   }
 
   // the second half of K hands its sums over through LDS (no load into LDS may still be on its way)
@@ -737,9 +750,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   }
 }
 
-template <int MW, int NT, int NB, typename TC, int EPI>
+template <int MW, int NT, int NB, typename TC, int EPI, int SPB = 1>
 static int launch_wide(const void* A, const void* W, void* C, int M, int N, int K, int up_offset, int parts,
                        const QkvRopeArgs& qa, hipStream_t stream) {
+  if (SPB > 1 && ((K >> 6) / parts) % SPB) return SA_ERR_ARG;      // whole groups of SPB stages
   constexpr int BM = 64 * MW;
   constexpr int COLS = EPI == EPI_SWIGLU ? 8 * NT : 16 * NT;
   constexpr size_t lds_bytes = (size_t)NB * (BM + 16 * NT) * 128;
@@ -748,7 +762,7 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
   if (EPI == EPI_QKV_ROPE) gx = ((qa.Hq + 2 * qa.Hk) * (qa.D >> 4) + NT - 1) / NT;
   dim3 grid(gx, parts, (M + BM - 1) / BM);
   if (grid.z > 65535 || parts < 1 || parts > 64) return SA_ERR_ARG;
-  auto kernel = gemm_wide_kernel<MW, NT, NB, TC, EPI>;
+  auto kernel = gemm_wide_kernel<MW, NT, NB, TC, EPI, SPB>;
   if (lds_bytes > 64 * 1024) {  // more dynamic LDS than a kernel gets without asking
     static bool allowed[64] = {};
     int dev = 0;
@@ -786,7 +800,8 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
 //   q/k/v + rotation + cache write (16 weight rows a workgroup, 32 where 16 would give more workgroups than
 //     compute units): K 2048, 3072 rows of W: 10.0 / 6.0 at one row, 10.2 / 8.4 at 32, 10.7 / 11.5 at 64, 13.6 / 17.3
 //     at 128; K 3072, 5120 rows: 15.8 / 16.5 at 48, 16.0 / 19.4 at 64, 21.8 / 28.5 at 128; K 4096, 6144 rows: 19.6 /
-//     19.5 at 48, 20.5 / 22.2 at 64, 26.8 / 33.5 at 128.
+//     19.5 at 48, 20.5 / 22.2 at 64, 26.8 / 33.5 at 128.  (Measured with one stage between two barriers; with two,
+//     see pick_wide, it is ahead from 40 rows on.)
 // 129 to 192 rows, against the BLAS library (and its SwiGLU pass): gate/up 22.7 / 30.6 at 160 rows and 24.4 / 31.0
 // at 192 with K 2048, 34.5 / 36.4 and 37.2 / 40.6 with K 3072, 62.2 / 65.8 and 64.0 / 68.7 with K 4096; down_proj
 // 18.4 / 25.7 and 20.8 / 26.9 (K 8192, 2048 rows), 26.0 / 27.6 and 29.2 / 58.5 (3072 rows), 57.4 / 83.4 and 64.9 /
@@ -800,7 +815,8 @@ static bool takes_wide(int M, int N, int K, int parts) {
   if (M < 1 || M > 256 || (K & 63) || parts < 1 || (K >> 6) % parts) return false;
   const int stages = (K >> 6) / parts;             // of a workgroup
   if (stages < 2) return false;
-  if (EPI == EPI_QKV_ROPE) return M >= 64 && M <= 128;
+  // q/k/v: from 64 rows; from 40 where the stages come in pairs (two of them between two barriers, see pick_wide)
+  if (EPI == EPI_QKV_ROPE) return M <= 128 && (M >= 64 || (M >= 40 && (stages & 1) == 0));
   // gate/up: beyond 192 rows only for matrices of up to 64 M elements, for which the library's fixed costs weigh most
   if (EPI == EPI_SWIGLU) return (K >= 3072 || M >= 16) && (M <= 192 || 2ll * N * K <= (64ll << 20));
   if (M > 192) return false;
@@ -823,9 +839,18 @@ static int pick_wide(const void* A, const void* W, void* C, int M, int N, int K,
 #define GO(MW, NT, NB) return launch_wide<MW, NT, NB, TC, EPI>(A, W, C, M, N, K, up_offset, parts, qa, stream)
   if constexpr (EPI == EPI_QKV_ROPE) {
     // few weight rows in all: 16 of them a workgroup, or 32 where that still gives every compute unit one
+    // With one product a wave and stage, the barrier and the trip through LDS are what a stage takes: up to
+    // 64 rows two stages go between two barriers, in a ring of eight (K 2048, 3072 rows of W: 8.1 us
+    // against 10.2 at 40 rows and 9.1 with gemm_mid_kernel, 8.9 against 10.9 at 64; K 3072, 5120 rows: 13.8
+    // against 15.8 at 40 and 15.6 with gemm_mid_kernel, 15.6 against 16.1 at 64; K 4096, 6144 rows: 17.9
+    // against 19.8 at 40 and 19.1, 20.2 against 20.5 at 64; no gain with more rows)
     const int tiles = (qa.Hq + 2 * qa.Hk) * (qa.D >> 4);
     const bool two = tiles > compute_units();
     if (M <= 64) {
+      if ((((K >> 6) / parts) & 1) == 0) {
+        if (two) return launch_wide<1, 2, 8, TC, EPI, 2>(A, W, C, M, N, K, up_offset, parts, qa, stream);
+        return launch_wide<1, 1, 8, TC, EPI, 2>(A, W, C, M, N, K, up_offset, parts, qa, stream);
+      }
       if (two) GO(1, 2, 6);
       GO(1, 1, 6);
     }

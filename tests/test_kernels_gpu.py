@@ -746,7 +746,11 @@ def test_gemm_split_k_parts_and_norm_that_adds_them(M, N, K, parts):
                                              # through LDS, 16 weight rows a workgroup, or 32 with more than 256 tiles
                                              # (an odd number of them: the last workgroup has one)
                                              (64, 32, 8, 64, 16, 2048), (100, 32, 8, 128, 16, 256), (64, 5, 1, 48, 16, 128),
-                                             (128, 40, 8, 128, 16, 192), (70, 3, 1, 80, 16, 128), (64, 85, 1, 48, 16, 128)])
+                                             (128, 40, 8, 128, 16, 192), (70, 3, 1, 80, 16, 128), (64, 85, 1, 48, 16, 128),
+                                             # 40 to 64 rows with the stages in pairs: two of them between two barriers; an odd
+                                             # number of stages at 64 rows: one
+                                             (40, 32, 8, 64, 16, 2048), (50, 5, 1, 48, 16, 256), (63, 85, 1, 48, 16, 128),
+                                             (64, 3, 1, 80, 16, 192), (48, 4, 2, 64, 16, 192), (57, 24, 8, 128, 16, 3072)])
 def test_qkv_rope_fused_equals_the_three_steps(M, Hq, Hk, D, ps, d):
     from serve_amd import ops
     P = 7 if M <= 64 else 20

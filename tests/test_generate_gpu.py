@@ -190,6 +190,40 @@ def test_graph_replays_equal_eager_steps(tmp_path):
     assert torch.equal(results[False], results[True])
 
 
+def test_large_vocabulary_through_steps_and_graphs(tmp_path):
+    """A vocabulary of more than 65,536 entries, where the head of 8 to 128 rows takes 256 weight rows a
+    workgroup: logits of decode steps of 12 requests (eager, and replayed from a graph) and of 50 wanted
+    rows of a prompt against the plain model."""
+    from serve_amd import ops
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.llama import LlamaConfig
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    from serve_amd.weights.loader import write_random_model
+    cfg = LlamaConfig(vocab_size=70001, hidden_size=128, intermediate_size=192, num_hidden_layers=1,
+                      num_attention_heads=4, num_key_value_heads=2, head_dim=32, rms_norm_eps=1e-5,
+                      rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True)
+    assert ops.gemm_takes_wide(12, cfg.vocab_size, cfg.hidden_size, 1) and ops.gemm_takes_wide(50, cfg.vocab_size, cfg.hidden_size, 1)
+    folder = write_random_model(os.path.join(str(tmp_path), "big_vocab"), cfg, seed=5, dtype=torch.bfloat16)
+    rng = random.Random(11)
+    toks = {k: util.random_tokens(rng, 30, cfg.vocab_size) for k in range(12)}
+    want = {k: util.plain_logits(folder, toks[k]) for k in toks}
+    for use_graphs in (False, True):
+        eng = Engine.from_folder(folder, EngineConfig(dtype="bfloat16", page_size=16, num_pages=40, max_context=64,
+                                                     max_requests=16, use_graphs=use_graphs))
+        for k in toks:
+            eng.runner.admit(k)
+        out = eng.step([Segment(k, toks[k][:20], list(range(20)) if k < 2 else [19]) for k in toks])   # 50 wanted rows
+        rows = [want[k][:20] if k < 2 else want[k][19:20] for k in toks]
+        util.assert_close(out.cpu().double(), torch.cat(rows), "bfloat16", "prompt rows over the large vocabulary")
+        for i in range(20, 30):
+            out = eng.step([Segment(k, [toks[k][i]], [0]) for k in toks])
+            util.assert_close(out.cpu().double(), torch.stack([want[k][i] for k in toks]), "bfloat16",
+                              f"decode step {i} over the large vocabulary (graphs {use_graphs})")
+            # the last column, the one beyond a multiple of 256, of 4 and of 2, is a value like the others
+            assert torch.isfinite(out[:, -1]).all()
+
+
 # ---------------------------------------------------------------------------------------------
 # each part alone
 # ---------------------------------------------------------------------------------------------

@@ -190,6 +190,37 @@ def test_graph_replays_equal_eager_steps(tmp_path):
     assert torch.equal(results[False], results[True])
 
 
+@pytest.mark.parametrize("live", [44, 64, 100])
+def test_many_rows_at_a_width_of_paired_stages(tmp_path, live):
+    """44, 64 and 100 requests decoded together by a model whose width is a whole number of pairs of 64
+    columns (256), where the fused q/k/v product of 40 to 128 rows takes both operands through LDS (two stages
+    between two barriers up to 64 rows): every logit of four decode steps, eager and replayed, against plain."""
+    from serve_amd import ops
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.config.llama import LlamaConfig
+    from serve_amd.engine.batch import Segment
+    from serve_amd.engine.engine import Engine
+    from serve_amd.weights.loader import write_random_model
+    cfg = LlamaConfig(vocab_size=300, hidden_size=256, intermediate_size=384, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-5,
+                      rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False)
+    folder = write_random_model(os.path.join(str(tmp_path), "wide256"), cfg, seed=9, dtype=torch.bfloat16,
+                                scales=util.SHARP_SCALES)
+    rng = random.Random(live)
+    toks = {k: util.random_tokens(rng, 5 + k % 7 + 4, cfg.vocab_size) for k in range(live)}
+    want = {k: util.plain_logits(folder, toks[k]) for k in toks}
+    for use_graphs in (False, True):
+        eng = Engine.from_folder(folder, EngineConfig(dtype="bfloat16", page_size=4, num_pages=live * 5, max_context=32,
+                                                     max_requests=128, use_graphs=use_graphs))
+        for k in toks:
+            eng.runner.admit(k)
+        eng.step([Segment(k, toks[k][:-4], []) for k in toks])
+        for i in range(4, 0, -1):
+            out = eng.step([Segment(k, [toks[k][-i]], [0]) for k in toks])
+            util.assert_close(out.cpu().double(), torch.stack([want[k][-i] for k in toks]), "bfloat16",
+                              f"{live} requests, decode step {5 - i} (graphs {use_graphs})")
+
+
 def test_large_vocabulary_through_steps_and_graphs(tmp_path):
     """A vocabulary of more than 65,536 entries, where the head of 8 to 128 rows takes 256 weight rows a
     workgroup: logits of decode steps of 12 requests (eager, and replayed from a graph) and of 50 wanted

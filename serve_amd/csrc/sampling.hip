@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void sample_partial_kernel(const float* __rest
                                                              const float* __restrict__ temperature,
                                                              const unsigned long long* __restrict__ keys,
                                                              float* __restrict__ part_v, int* __restrict__ part_i,
-                                                             int V, int chunk) {
+                                                             int V, int chunk, int by_four) {
   __shared__ float sv[4];
   __shared__ int si[4];
   const int r = blockIdx.y;
@@ -43,14 +43,28 @@ __global__ __launch_bounds__(256) void sample_partial_kernel(const float* __rest
   const int hi = min(V, lo + chunk);
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
-    float v = row[i];
+  auto score = [&](float v, int i) __attribute__((always_inline)) {
     if (!greedy) {
       const unsigned int bits = (unsigned int)(mix64(key ^ (unsigned long long)i) >> 41);
       const float u = ((float)bits + 0.5f) * (1.0f / 8388608.0f);
       v = v * inv_t - logf(-logf(u));
     }
     take_better(bv, bi, v, i);
+  };
+  if (by_four) {
+    // rows and chunks begin on 16-byte boundaries and hold whole groups of four: 16 bytes a load
+    const float4* row4 = reinterpret_cast<const float4*>(row + lo);
+    const int n4 = (hi - lo) >> 2;
+    for (int j = threadIdx.x; j < n4; j += blockDim.x) {
+      const float4 q = row4[j];
+      const int i = lo + 4 * j;
+      score(q.x, i);
+      score(q.y, i + 1);
+      score(q.z, i + 2);
+      score(q.w, i + 3);
+    }
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) score(row[i], i);
   }
 #pragma unroll
   for (int o = SA_WAVE / 2; o > 0; o >>= 1) {
@@ -102,9 +116,13 @@ extern "C" int sa_sample(const float* logits, const float* temperature, const un
   if (R <= 0) return 0;
   if (V <= 0 || R > 65535 || !part_v || !part_i) return SA_ERR_ARG;
   const int nchunks = sa_sample_chunks(V);
-  const int chunk = (V + nchunks - 1) / nchunks;
+  int chunk = (V + nchunks - 1) / nchunks;
+  // a vocabulary of whole groups of four from an aligned address is read 16 bytes a lane (chunks of whole
+  // groups too; the last chunks may then be shorter or empty, which the second stage does not mind)
+  const int by_four = (V & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0;
+  if (by_four) chunk = (chunk + 3) & ~3;
   hipLaunchKernelGGL(sample_partial_kernel, dim3(nchunks, R), dim3(256), 0, stream, logits, temperature, keys,
-                     part_v, part_i, V, chunk);
+                     part_v, part_i, V, chunk, by_four);
   SA_LAUNCH_CHECK();
   hipLaunchKernelGGL(sample_final_kernel, dim3(R), dim3(64), 0, stream, part_v, part_i, out, nchunks);
   SA_LAUNCH_CHECK();

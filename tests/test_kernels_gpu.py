@@ -424,17 +424,24 @@ def test_silu_mul(dtype):
     assert out[0].abs().max().item() == 0
 
 
-def test_sample_greedy_and_ties():
+@pytest.mark.parametrize("V,shift", [(1000, 0), (1001, 0), (1000, 1), (6152, 0), (128256, 0), (70001, 0)])
+def test_sample_greedy_and_ties(V, shift):
+    """One chunk and many; vocabularies of whole groups of four from an aligned address (read 16 bytes a lane,
+    6152 being one whose chunks are rounded up so that the last one is short) and others (a width that is no
+    multiple of four, an address four bytes off)."""
     from serve_amd import ops
-    R, V = 7, 1000
-    logits = rnd((R, V), torch.float32, 10)
+    R = 7
+    flat = rnd((R * V + shift,), torch.float32, 10)
+    logits = flat[shift:].view(R, V)
     logits[2, 400] = logits[2, 900] = 50.0             # tie -> lowest index
-    logits[3, 999] = 60.0                              # last entry
+    logits[3, V - 1] = 60.0                            # last entry
     logits[4, 0] = 60.0
+    logits[5, V - 2] = logits[5, V - 1] = 55.0         # a tie at the very end
     out = torch.empty(R, dtype=torch.int32, device=DEV)
     ops.sample(logits, None, None, out)
     want = torch.argmax(logits, dim=-1)
     want[2] = 400
+    want[5] = V - 2
     assert out.tolist() == want.tolist()
 
 

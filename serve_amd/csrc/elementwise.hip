@@ -20,11 +20,41 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
   for (int i = threadIdx.x; i < d; i += blockDim.x) x[(size_t)t * d + i] = to_float(table[row + i]);
 }
 
+// bf16 rows of whole groups of eight from aligned addresses: 16 bytes a lane in, two times 16 out
+__global__ __launch_bounds__(256) void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int* __restrict__ tokens,
+                                                            const int* __restrict__ src_row, const int* __restrict__ prev,
+                                                            float* __restrict__ x, int d, int V) {
+  const int t = blockIdx.x;
+  int tok = tokens[t];
+  if (src_row && src_row[t] >= 0) tok = prev[src_row[t]];
+  tok = min(max(tok, 0), V - 1);
+  const bf16_t* row = table + (size_t)tok * (size_t)d;
+  float* out = x + (size_t)t * d;
+  for (int i = threadIdx.x * 8; i < d; i += blockDim.x * 8) {
+    const uint4 v = *reinterpret_cast<const uint4*>(row + i);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float f[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      f[2 * k] = bf16_bits_to_float(w[k] & 0xffffu);
+      f[2 * k + 1] = bf16_bits_to_float(w[k] >> 16);
+    }
+    *reinterpret_cast<float4*>(out + i) = make_float4(f[0], f[1], f[2], f[3]);
+    *reinterpret_cast<float4*>(out + i + 4) = make_float4(f[4], f[5], f[6], f[7]);
+  }
+}
+
 extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, const int* src_row,
                         const int* prev, float* x, int T, int d, int V, hipStream_t stream) {
   if (T <= 0) return 0;
   if (d <= 0 || V <= 0 || (src_row && !prev)) return SA_ERR_ARG;
   dim3 grid(T), block(256);
+  if (table_dtype == SA_BF16 && (d & 7) == 0 && ((uintptr_t)table & 15) == 0 && ((uintptr_t)x & 15) == 0) {
+    hipLaunchKernelGGL(embed_bf16x8_kernel, grid, block, 0, stream, (const bf16_t*)table, tokens, src_row, prev, x,
+                       d, V);
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
   if (table_dtype == SA_F32)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, src_row, prev,
                        x, d, V);

@@ -26,9 +26,11 @@ def tol(dtype):
 
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_embed(dtype):
+@pytest.mark.parametrize("d", [72, 76, 2048 + 8])
+def test_embed(dtype, d):
+    """Widths of whole groups of eight (bf16 rows then go 16 bytes a lane, several trips at 2,056) and 76, which is none."""
     from serve_amd import ops
-    V, d = 301, 72
+    V = 301
     table = rnd((V, d), DT[dtype], 0)
     tokens = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
     out = torch.empty((5, d), dtype=torch.float32, device=DEV)

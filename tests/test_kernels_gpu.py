@@ -693,6 +693,82 @@ def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
     assert not ops.gemm_takes_wide(257, N, K, parts) and not ops.gemm_takes_wide(M, N, K + 8, parts)
 
 
+def test_random_sizes_through_the_few_row_products():
+    """400 random cases of rows, widths, inner sizes, parts and head layouts through the products for few rows
+    (plain, fp32 parts, gate/up with SwiGLU, the head over a large vocabulary, the fused q/k/v) against float64:
+    whatever kernel and workgroup shape the dispatch picks for a size, the numbers are the product's."""
+    import random
+    from serve_amd import ops
+    checked, wide = 0, 0
+    for seed in range(400):
+        rng = random.Random(seed)
+        torch.manual_seed(seed)
+        kind = rng.choice(["plain", "parts", "swiglu", "qkv", "head"])
+        M = rng.choice([1, 2, 3, 8, 9, 16, 17, 31, 33, 40, 41, 48, 63, 64, 65, 80, 100, 127, 128, 129, 160, 192, 193, 255, 256])
+        K = 64 * rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64]) + rng.choice([0, 0, 0, 8, 32])
+        what = f"seed {seed}: {kind} M={M} K={K}"
+        if kind == "qkv":
+            M = min(M, 128)
+            D = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+            Hk = rng.choice([1, 2, 3, 8])
+            Hq = Hk * rng.choice([1, 2, 4, 5])
+            if rng.random() < 0.2:
+                Hq, Hk, D = 85, 1, 48                      # more tiles of 16 weight rows than compute units
+            ps = rng.choice([4, 8, 16, 32])
+            P = -(-M // ps) + 3
+            a = torch.randn(M, K, device=DEV, dtype=torch.bfloat16)
+            w = torch.randn((Hq + 2 * Hk) * D, K, device=DEV, dtype=torch.bfloat16) * 0.05
+            k1 = torch.zeros(P, Hk, ps, D, device=DEV, dtype=torch.bfloat16)
+            v1 = torch.zeros(P, Hk, D, ps, device=DEV, dtype=torch.bfloat16)
+            if not ops.qkv_rope_available(a, w, k1, D, D, False):
+                continue
+            pos = torch.randint(0, 100000, (M,), device=DEV, dtype=torch.int32)
+            inv = (1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+            slots = torch.randperm(P * ps, device=DEV)[:M].to(torch.int32)
+            slots[rng.randrange(M)] = -1
+            q = torch.empty(M, Hq * D, device=DEV, dtype=torch.bfloat16)
+            ops.qkv_rope_bf16(a, w, q, pos, inv, slots, k1, v1, Hq, Hk, D, ps)
+            x = (a.double() @ w.double().T).view(M, Hq + 2 * Hk, D)
+            bound = dict(atol=2e-2 * max(1.0, x.abs().max().item()), rtol=1e-2)
+            torch.testing.assert_close(q.double(), rope_ref(x[:, :Hq], pos, inv, D, False).reshape(M, Hq * D), msg=what, **bound)
+            ok = slots >= 0
+            page, off = (slots[ok] // ps).long(), (slots[ok] % ps).long()
+            torch.testing.assert_close(k1.double()[page, :, off, :], rope_ref(x[:, Hq:Hq + Hk], pos, inv, D, False)[ok], msg=what, **bound)
+            torch.testing.assert_close(v1.double()[page, :, :, off], x[:, Hq + Hk:][ok], msg=what, **bound)
+            checked += 1
+            continue
+        N = rng.choice([8, 40, 64, 100, 520, 1000, 2048, 2050, 4100, 8192, 8200, 12296, 33001, 65536, 65543, 70000])
+        if kind == "head":
+            N, K = rng.choice([65536, 65537, 65600, 66000, 70001]), min(K, 512)
+        if N * K > 40e6:
+            K = 64 * rng.choice([2, 4])
+        a = torch.randn(M, K, device=DEV, dtype=torch.bfloat16)
+        if kind == "swiglu":
+            if M > ops.SKINNY_MAX_ROWS and not ops.gemm_takes_wide(M, N, K, 1, swiglu=True):
+                continue
+            w = torch.randn(2 * N, K, device=DEV, dtype=torch.bfloat16) * 0.05
+            out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+            ops.swiglu_bf16(a, w, out)
+            gu = a.double() @ w.double().T
+            want = torch.nn.functional.silu(gu[:, :N]) * gu[:, N:]
+            torch.testing.assert_close(out.double(), want, atol=2e-2 * max(1.0, want.abs().max().item()), rtol=1e-2, msg=what + f" N={N}")
+            wide += ops.gemm_takes_wide(M, N, K, 1, swiglu=True)
+        else:
+            parts = rng.choice([2, 4, 8]) if kind == "parts" else 1
+            if K % 64 or (K // 64) % parts:
+                parts = 1
+            if M > ops.SKINNY_MAX_ROWS and not ops.gemm_takes_wide(M, N, K, parts):
+                continue
+            w = torch.randn(N, K, device=DEV, dtype=torch.bfloat16) * 0.05
+            out = torch.full((parts, M, N) if parts > 1 else (M, N), float("nan"), device=DEV, dtype=torch.float32)
+            ops.gemm_bf16_skinny(a, w, out)
+            got = out.double().sum(0) if parts > 1 else out.double()
+            torch.testing.assert_close(got, a.double() @ w.double().T, atol=3e-4 * K ** 0.5, rtol=1e-4, msg=what + f" N={N} parts={parts}")
+            wide += ops.gemm_takes_wide(M, N, K, parts)
+        checked += 1
+    assert checked >= 300 and wide >= 60, (checked, wide)
+
+
 def test_kernels_refuse_what_they_do_not_take():
     from serve_amd import ops
     a = rnd((4, 12), torch.bfloat16, 1)

@@ -693,6 +693,53 @@ def test_products_with_both_operands_in_lds(kind, M, N, K, parts):
     assert not ops.gemm_takes_wide(257, N, K, parts) and not ops.gemm_takes_wide(M, N, K + 8, parts)
 
 
+def test_random_shapes_segments_windows_and_splits_through_attention():
+    """150 random cases through the attention kernels of both paths (single tokens with the key range whole, cut
+    across workgroups or inside one; prompt portions; both in one step; the float32 kernels), head sizes 16 to
+    128, page sizes 4 to 64, contexts on both sides of page and block edges, windows, now and then with every
+    unowned page full of NaN, against dense float64 softmax."""
+    import random
+    from serve_amd import ops
+    done = {}
+    for seed in range(150):
+        rng = random.Random(seed)
+        D = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+        Hk = rng.choice([1, 2, 3, 8])
+        G = rng.choice([1, 2, 4, 5, 8])
+        ps = rng.choice([4, 8, 12, 16, 32, 64])
+        kind = rng.choice(["decode", "decode", "prompt", "mixed", "f32decode", "f32tiled"])
+        nseg = rng.choice([1, 2, 3, 5, 9, 17, 40])
+        ctx = lambda: rng.choice([0, 1, 3, 15, 16, 17, 63, 64, 100, 255, 256, 257, 700, 1500])
+        window = rng.choice([None, None, None, 16, 100])
+        splits, inwg, kernel, dtype = 1, False, "mfma", "bfloat16"
+        if kind == "decode":
+            segs = [(ctx(), 1) for _ in range(nseg)]
+            splits = rng.choice([1, 1, 2, 4, 8, 16])
+            inwg = splits == 1 and rng.random() < 0.5
+        elif kind == "prompt":
+            segs = [(ctx(), rng.choice([2, 3, 16, 17, 33, 64, 100, 130, 300])) for _ in range(min(nseg, 5))]
+            splits = rng.choice([1, 1, 2, 4])
+        elif kind == "mixed":
+            segs = [(ctx(), 1) for _ in range(nseg)] + [(ctx(), rng.choice([2, 5, 40, 129])) for _ in range(rng.choice([1, 2, 3]))]
+        elif kind == "f32decode":
+            segs = [(ctx(), 1) for _ in range(nseg)]
+            kernel, dtype, splits = "decode_f32", "float32", rng.choice([1, 2, 4, 8])
+        else:
+            segs = [(ctx(), rng.choice([1, 2, 16, 40, 64, 65, 200])) for _ in range(min(nseg, 6))]
+            kernel, dtype, splits = "tiled", "float32", rng.choice([1, 1, 2, 4])
+        poison = rng.random() < 0.3 and window is None
+        try:
+            attention_case(dtype, Hk * G, Hk, D, ps, segs, seed=seed, window=window, kernel=kernel, splits=splits,
+                           in_workgroup=inwg, poison=poison)
+        except ops.KernelError:
+            continue                                        # a combination that the kernel refuses
+        except AssertionError as e:
+            raise AssertionError(f"seed {seed}: {kind} D={D} Hq={Hk * G} Hk={Hk} ps={ps} window={window} splits={splits} "
+                                 f"in_workgroup={inwg} poison={poison} segs={segs}: {e}") from None
+        done[kind] = done.get(kind, 0) + 1
+    assert sum(done.values()) >= 120 and len(done) == 5, done
+
+
 def test_random_sizes_through_the_few_row_products():
     """400 random cases of rows, widths, inner sizes, parts and head layouts through the products for few rows
     (plain, fp32 parts, gate/up with SwiGLU, the head over a large vocabulary, the fused q/k/v) against float64:
